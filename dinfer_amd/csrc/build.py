@@ -36,6 +36,8 @@ SOURCES = {
     "latent": "latent.hip",
     "grouped": "grouped.hip",
     "delta": "delta.hip",
+    "decay": "decay.hip",
+    "streams": "streams.hip",
     "sampling": "sampling.hip",
     "ceilings": "ceilings.hip",
     "host": "host/api.cpp",

@@ -1,0 +1,323 @@
+// Linear recurrences with a scalar decay: per request and head one matrix S [D, V] in float,
+//
+//   per token:   S <- a_t S + c_t k_t v_t^T;   o_t = S^T q_t
+//
+// with a_t in (0, 1] a decay (one a head, or one a head and token) and c_t an optional step size a head and token.
+// Two mixers are this recurrence with different things around it:
+//
+//   retention       q, k rotated by the position, k scaled; a fixed decay a head; no step size
+//   state space     q = C_t, k = B_t (shared by the heads of a group), v = x_t; a_t = exp(-exp(A) dt_t), c_t = dt_t;
+//                   x, B and C come out of a short causal convolution with bias and silu
+//
+//   rot_widen          one workgroup a token: q and k heads rotated (pairs (i, i + rot/2) of the first rot entries) by the
+//                      table row of the token's position, k times a scale, v widened; float out
+//   conv_silu          a thread a (token, channel): taps over the step's rows and the request's stored inputs, bias, silu;
+//                      the threads behind the channels make dt = softplus(. + bias) and exp(-exp(A) dt) of every head
+//   decay_recurrence   token by token, one request, one head and 8 columns of S a workgroup: the 32 lanes of half a wave
+//                      share a column and own a strip of its rows; 16 tokens' operands wait in LDS while the next 16 are
+//                      on their way in registers. Serves single decoded rows (the whole state in and out once) and
+//                      prompt portions of any length
+//   gated_group_norm   (y + skip_h x) * silu(z), then divided by the root mean square of its group of columns, times a
+//                      gain a column; or the gate after the norm; one workgroup a (token, group)
+//
+// S is stored transposed, [slot][head][V][D], as the delta rule's state is: a thread's strip is contiguous.
+// A request whose step starts at position 0 starts from S = 0 and zero stored inputs, whatever its slot held.
+#include "common.cuh"
+
+using namespace dinfer;
+
+namespace {
+
+constexpr int CH = 16;          // tokens of a chunk in the token-by-token recurrence
+constexpr int COLS = 8;         // columns of S a workgroup
+constexpr int MAX_TAPS = 16;
+
+__device__ __forceinline__ int request_of(const int32_t* __restrict__ cu, int num_reqs, int t) {
+  int lo = 0, hi = num_reqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// work row: q (H D) | k (H D) | v (H V), float
+template <class S>
+__global__ void __launch_bounds__(256) rot_widen_kernel(const S* __restrict__ proj, int64_t ld, int64_t q_off,
+                                                        int64_t k_off, int64_t v_off, const int32_t* __restrict__ pos,
+                                                        const float* __restrict__ cos_sin, int rot, float k_scale,
+                                                        float* __restrict__ work, int64_t ldw, int H, int D, int V) {
+  const int64_t t = blockIdx.x;
+  const S* row = proj + t * ld;
+  float* wr = work + t * ldw;
+  const int half = rot / 2;
+  const float* cs = (cos_sin && rot > 0) ? cos_sin + (int64_t)pos[t] * rot : nullptr;
+  const int hd = H * D;
+  for (int c = threadIdx.x; c < 2 * hd; c += blockDim.x) {
+    const bool is_k = c >= hd;
+    const int e = is_k ? c - hd : c;
+    const int d = e % D;
+    const S* src = row + (is_k ? k_off : q_off);
+    float y = to_f32(src[e]);
+    if (cs && d < rot) {
+      const bool first = d < half;
+      const int i = first ? d : d - half;
+      const float other = to_f32(src[first ? e + half : e - half]);
+      y = first ? rotated_first(y, other, cs[i], cs[half + i]) : rotated_second(other, y, cs[i], cs[half + i]);
+    }
+    wr[c] = is_k ? y * k_scale : y;
+  }
+  for (int c = threadIdx.x; c < H * V; c += blockDim.x) wr[2 * hd + c] = to_f32(row[v_off + c]);
+}
+
+// work row: the C channels after convolution, bias and silu | dt (H) | decay (H), float
+template <class S>
+__global__ void __launch_bounds__(256) conv_silu_kernel(
+    const S* __restrict__ proj, int64_t ld, int64_t x_off, int64_t dt_off, const float* __restrict__ taps,
+    const float* __restrict__ bias, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    const S* __restrict__ conv_state, const int32_t* __restrict__ slots, const int32_t* __restrict__ cu,
+    const int32_t* __restrict__ seq_lens, float* __restrict__ work, int64_t ldw, int num_reqs, int C, int H, int K) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C + H) return;
+  const S* row = proj + (int64_t)t * ld;
+  float* wr = work + (int64_t)t * ldw;
+  if (c >= C) {
+    const int h = c - C;
+    const float dt = softplus_f(to_f32(row[dt_off + h]) + dt_bias[h]);
+    wr[C + h] = dt;
+    wr[C + H + h] = expf(-expf(a_log[h]) * dt);
+    return;
+  }
+  const int b = request_of(cu, num_reqs, t);
+  const int i = t - cu[b];                                   // index of the token in its request's rows of this step
+  const int start = seq_lens[b] - (cu[b + 1] - cu[b]);       // position of the request's first row of this step
+  const S* old = (K > 1 && start > 0) ? conv_state + (int64_t)slots[b] * C * (K - 1) : nullptr;
+  float acc = bias ? bias[c] : 0.f;
+  for (int j = K - 1; j >= 0; --j) {                         // the oldest input first
+    float x = 0.f;
+    if (i - j >= 0) x = to_f32(row[x_off + c - (int64_t)j * ld]);
+    else if (old) x = to_f32(old[(int64_t)c * (K - 1) + (K - 1 + i - j)]);
+    acc = __builtin_fmaf(taps[(int64_t)c * K + (K - 1 - j)], x, acc);
+  }
+  wr[c] = silu_f(acc);
+}
+
+// A lane's value plus that of the lane a DPP pattern pairs it with (full-rate vector instructions, no LDS).
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// The sum over 32 lanes (two DPP rows of 16), in every lane of them.
+__device__ __forceinline__ float half_wave_sum(float v) {
+  v = dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  v = dpp_add<0x141>(v);   // row_half_mirror
+  v = dpp_add<0x140>(v);   // row_mirror
+  return v + __shfl_xor(v, 16, WAVE);
+}
+
+struct Operands {
+  const float* q; int64_t ldq;        // [T, G D]
+  const float* k; int64_t ldk;        // [T, G D]
+  const float* v; int64_t ldv;        // [T, H V]
+  const float* decay; int64_t ldd;    // [T, H], or [H] with ldd = 0
+  const float* gain; int64_t ldg;     // [T, H] or null
+};
+
+// One request, one head and COLS columns of S a workgroup; a thread owns RPT consecutive rows of a column (D <= 32 RPT).
+template <int RPT>
+__global__ void __launch_bounds__(256) decay_recurrence_kernel(Operands p, float* __restrict__ state,
+                                                               const int32_t* __restrict__ slots,
+                                                               const int32_t* __restrict__ cu,
+                                                               const int32_t* __restrict__ seq_lens,
+                                                               float* __restrict__ out, int64_t ld_out, int G, int H,
+                                                               int D, int V) {
+  constexpr int DP = 32 * RPT;
+  __shared__ __attribute__((aligned(16))) float ks[CH][DP];
+  __shared__ __attribute__((aligned(16))) float qs[CH][DP];
+  __shared__ float vs[CH][COLS];
+  __shared__ float as[CH];
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int rg = tid & 31, cj = tid >> 5;
+  const int j = blockIdx.z * COLS + cj;
+  const int t0 = cu[b], n = cu[b + 1] - t0;
+  const int start = seq_lens[b] - n;
+  const int g = h / (H / G);
+  const bool col_ok = j < V;
+  float* sp = state + ((((int64_t)slots[b] * H + h) * V + (col_ok ? j : 0)) * D) + rg * RPT;
+  float S[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) S[i] = (start > 0 && col_ok && rg * RPT + i < D) ? sp[i] : 0.f;
+
+  // what a thread carries of the next chunk: entries of k and of q, one of v (times its step size), one decay
+  constexpr int PK = (CH * DP) / 256;
+  float pk[PK], pq[PK], pv = 0.f, pa = 0.f;
+  auto fetch = [&](int ct) {
+#pragma unroll
+    for (int e = 0; e < PK; ++e) {
+      const int idx = tid + e * 256;
+      const int tok = idx / DP, d = idx % DP;
+      const bool ok = ct + tok < n && d < D;
+      const int64_t t = t0 + ct + tok;
+      pk[e] = ok ? p.k[t * p.ldk + g * D + d] : 0.f;
+      pq[e] = ok ? p.q[t * p.ldq + g * D + d] : 0.f;
+    }
+    if (tid < CH * COLS) {
+      const int tok = tid / COLS, c = tid % COLS;
+      const int col = blockIdx.z * COLS + c;
+      const int64_t t = t0 + ct + tok;
+      pv = 0.f;
+      if (ct + tok < n && col < V) {
+        pv = p.v[t * p.ldv + h * V + col];
+        if (p.gain) pv *= p.gain[t * p.ldg + h];
+      }
+    }
+    if (tid < CH) pa = ct + tid < n ? p.decay[(int64_t)(t0 + ct + tid) * p.ldd + h] : 1.f;
+  };
+  fetch(0);
+  for (int ct = 0; ct < n; ct += CH) {
+    __syncthreads();  // the chunk before has been consumed
+#pragma unroll
+    for (int e = 0; e < PK; ++e) {
+      const int idx = tid + e * 256;
+      ks[idx / DP][idx % DP] = pk[e];
+      qs[idx / DP][idx % DP] = pq[e];
+    }
+    if (tid < CH * COLS) vs[tid / COLS][tid % COLS] = pv;
+    if (tid < CH) as[tid] = pa;
+    __syncthreads();
+    if (ct + CH < n) fetch(ct + CH);  // in flight while this chunk is worked through
+    const int m = n - ct < CH ? n - ct : CH;
+    for (int tok = 0; tok < m; ++tok) {
+      const float a = as[tok], vt = vs[tok][cj];
+      float o0 = 0.f, o1 = 0.f;   // two chains: a fixed order all the same
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        S[i] = __builtin_fmaf(ks[tok][rg * RPT + i], vt, a * S[i]);
+        if (i & 1) o1 = __builtin_fmaf(S[i], qs[tok][rg * RPT + i], o1);
+        else o0 = __builtin_fmaf(S[i], qs[tok][rg * RPT + i], o0);
+      }
+      const float o = half_wave_sum(o0 + o1);
+      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * V + j] = o;
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+      if (rg * RPT + i < D) sp[i] = S[i];
+  }
+}
+
+// gate_first: out[t, col_off + c] = u / sqrt(mean over c's group of u^2 + eps) * w[c],  u = (y[t, c] + skip[c / V] x[t, c]) * silu(z[t, c]);
+// else the gate comes after the norm: u = y + skip x, out = u / sqrt(mean u^2 + eps) * w[c] * silu(z[t, c])
+template <class S>
+__global__ void __launch_bounds__(256) gated_group_norm_kernel(const float* __restrict__ y, int64_t ld_y,
+                                                               const float* __restrict__ x, int64_t ld_x,
+                                                               const float* __restrict__ skip, int V,
+                                                               const S* __restrict__ z, int64_t ld_z, int64_t z_off,
+                                                               const float* __restrict__ w, S* __restrict__ out,
+                                                               int64_t ld_out, int64_t col_off, int group, float eps,
+                                                               float out_scale, int gate_first) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const int c0 = blockIdx.y * group;
+  auto value = [&](int c) {
+    float u = y[t * ld_y + c];
+    if (skip) u = __builtin_fmaf(skip[c / V], x[t * ld_x + c], u);
+    return gate_first ? u * silu_f(to_f32(z[t * ld_z + z_off + c])) : u;
+  };
+  float ss = 0.f;
+  for (int c = c0 + threadIdx.x; c < c0 + group; c += 256) {
+    const float u = value(c);
+    ss = __builtin_fmaf(u, u, ss);
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)group + eps);
+  for (int c = c0 + threadIdx.x; c < c0 + group; c += 256) {
+    float r = value(c) * inv * (w ? w[c] : 1.f) * out_scale;
+    if (!gate_first) r *= silu_f(to_f32(z[t * ld_z + z_off + c]));
+    out[t * ld_out + col_off + c] = from_f32<S>(r);
+  }
+}
+
+}  // namespace
+
+// proj [T, ld] in the step's dtype: H heads of q (size D) from column q_off, of k from k_off, H heads of v (size V) from
+// v_off. cos_sin float [positions, rot] = [cos | sin] (null or rot 0: no rotation). work [T, ldw] float:
+// q (H D) | k (H D) | v (H V), k times k_scale.
+extern "C" int dinfer_rot_widen(int dtype, const void* proj, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off,
+                                const int32_t* positions, const float* cos_sin, int rot, float k_scale, float* work,
+                                int64_t ldw, int64_t tokens, int H, int D, int V, hipStream_t stream) {
+  if (tokens <= 0) return OK;
+  if (H <= 0 || D <= 0 || V <= 0 || rot < 0 || rot > D || rot % 2 || tokens > 0x7fffffff ||
+      ldw < 2 * (int64_t)H * D + (int64_t)H * V)
+    return ERR_BAD_SHAPE;
+  DINFER_DISPATCH_DTYPE(dtype, {
+    rot_widen_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)proj, ld, q_off, k_off, v_off, positions, cos_sin,
+                                                              rot, k_scale, work, ldw, H, D, V);
+  });
+  return launch_status();
+}
+
+// proj [T, ld]: C channels from column x_off (they pass the convolution), H step-size logits from dt_off. taps [C, K]
+// float, the last column the current token's; bias [C] float or null; a_log, dt_bias [H] float. conv_state
+// [slots, C, K - 1] in the step's dtype (unused with K = 1). work [T, ldw] float, ldw >= C + 2 H.
+extern "C" int dinfer_conv_silu(int dtype, const void* proj, int64_t ld, int64_t x_off, int64_t dt_off, const float* taps,
+                                const float* bias, const float* a_log, const float* dt_bias, const void* conv_state,
+                                const int32_t* state_slots, const int32_t* cu_seqlens, const int32_t* seq_lens,
+                                float* work, int64_t ldw, int num_reqs, int64_t tokens, int C, int H, int K,
+                                hipStream_t stream) {
+  if (tokens <= 0 || num_reqs <= 0) return OK;
+  if (C <= 0 || H <= 0 || K <= 0 || tokens > 0x7fffffff || ldw < (int64_t)C + 2 * H) return ERR_BAD_SHAPE;
+  if (K > MAX_TAPS) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tokens, (unsigned)((C + H + 255) / 256));
+  DINFER_DISPATCH_DTYPE(dtype, {
+    conv_silu_kernel<S><<<grid, 256, 0, stream>>>((const S*)proj, ld, x_off, dt_off, taps, bias, a_log, dt_bias,
+                                                  (const S*)conv_state, state_slots, cu_seqlens, seq_lens, work, ldw,
+                                                  num_reqs, C, H, K);
+  });
+  return launch_status();
+}
+
+// q, k [T, G D], v [T, H V] float; decay [T, H] (ld_decay its row stride) or [H] (ld_decay 0); gain [T, H] or null.
+// state [slots, H, V, D] float (S transposed); out [T, ld_out] float, head h at column h V.
+extern "C" int dinfer_decay_recurrence(const float* q, int64_t ldq, const float* k, int64_t ldk, const float* v,
+                                       int64_t ldv, const float* decay, int64_t ld_decay, const float* gain,
+                                       int64_t ld_gain, float* state, const int32_t* state_slots,
+                                       const int32_t* cu_seqlens, const int32_t* seq_lens, float* out, int64_t ld_out,
+                                       int num_reqs, int G, int H, int D, int V, hipStream_t stream) {
+  if (num_reqs <= 0) return OK;
+  if (G <= 0 || H <= 0 || H % G || D <= 0 || V <= 0 || num_reqs > 0x7fffffff || H > 65535 || !decay) return ERR_BAD_SHAPE;
+  if (D > 256) return ERR_UNSUPPORTED;
+  Operands p{q, ldq, k, ldk, v, ldv, decay, ld_decay, gain, ld_gain};
+  const dim3 grid((unsigned)num_reqs, (unsigned)H, (unsigned)((V + COLS - 1) / COLS));
+#define DECAY_REC(R_) \
+  decay_recurrence_kernel<R_><<<grid, 256, 0, stream>>>(p, state, state_slots, cu_seqlens, seq_lens, out, ld_out, G, H, D, V)
+  if (D <= 32) DECAY_REC(1);
+  else if (D <= 64) DECAY_REC(2);
+  else if (D <= 128) DECAY_REC(4);
+  else DECAY_REC(8);
+#undef DECAY_REC
+  return launch_status();
+}
+
+// y [T, ld_y] float, `groups` groups of `group` columns each; x [T, ld_x] float with skip [groups * group / V] (both or
+// neither); z [T, ld_z] in the step's dtype, the gate's columns from z_off; w [groups * group] float or null.
+extern "C" int dinfer_gated_group_norm(int dtype, const float* y, int64_t ld_y, const float* x, int64_t ld_x,
+                                       const float* skip, int V, const void* z, int64_t ld_z, int64_t z_off,
+                                       const float* w, void* out, int64_t ld_out, int64_t col_off, int64_t tokens,
+                                       int groups, int group, float eps, float out_scale, int gate_first,
+                                       hipStream_t stream) {
+  if (tokens <= 0) return OK;
+  if (groups <= 0 || group <= 0 || groups > 65535 || tokens > 0x7fffffff || (skip && (!x || V <= 0))) return ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)tokens, (unsigned)groups);
+  DINFER_DISPATCH_DTYPE(dtype, {
+    gated_group_norm_kernel<S><<<grid, 256, 0, stream>>>(y, ld_y, x, ld_x, skip, V, (const S*)z, ld_z, z_off, w, (S*)out,
+                                                         ld_out, col_off, group, eps, out_scale, gate_first);
+  });
+  return launch_status();
+}

@@ -123,10 +123,13 @@ __global__ void __launch_bounds__(256) embedding_to_kernel(const int32_t* __rest
   for (int64_t i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_f32<O>(to_f32(src[i]) * scale);
 }
 
-// Activations of one argument: 0 silu, 1 the square of relu, 2 gelu in its tanh form.
+// Activations of one argument: 0 silu, 1 the square of relu, 2 gelu in its tanh form, 3 gelu with the error function,
+// 4 the logistic function.
 __device__ __forceinline__ float act1(float z, int act) {
   if (act == 0) return z / (1.f + expf(-z));
   if (act == 1) { const float r = fmaxf(z, 0.f); return r * r; }
+  if (act == 3) return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
+  if (act == 4) return 1.f / (1.f + expf(-z));
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
@@ -136,6 +139,14 @@ __global__ void __launch_bounds__(256) act_kernel(const S* __restrict__ in, int6
   const int64_t t = blockIdx.y;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
     out[t * ld_out + i] = from_f32<S>(act1(to_f32(in[t * ld_in + i]), act));
+}
+
+template <class S>
+__global__ void __launch_bounds__(256) gate_kernel(S* __restrict__ x, int64_t ld_x, const S* __restrict__ g, int64_t ld_g,
+                                                   int64_t n, int act) {
+  const int64_t t = blockIdx.y;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    x[t * ld_x + i] = from_f32<S>(to_f32(x[t * ld_x + i]) * act1(to_f32(g[t * ld_g + i]), act));
 }
 
 }  // namespace
@@ -231,11 +242,28 @@ extern "C" int dinfer_embedding_to(int table_dtype, int out_dtype, const int32_t
   return launch_status();
 }
 
-// out[t, i] = act(in[t, i]) for i < n (in place allowed). act: 0 silu, 1 relu squared, 2 gelu (tanh form).
+// x[t, i] *= act(g[t, i]) for i < n: a gate on a block of columns (x and g point at the first column of theirs).
+extern "C" int dinfer_gate(int dtype, int act, void* x, int64_t ld_x, const void* g, int64_t ld_g, int64_t tokens,
+                           int64_t n, hipStream_t stream) {
+  if (tokens <= 0 || n <= 0) return OK;
+  if (act < 0 || act > 4) return ERR_UNSUPPORTED;
+  if (ld_x < n || ld_g < n) return ERR_BAD_SHAPE;
+  for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
+    const int64_t nt = tokens - t0 < 65535 ? tokens - t0 : 65535;
+    const dim3 grid((unsigned)((n + 1023) / 1024 < 64 ? (n + 1023) / 1024 : 64), (unsigned)nt);
+    DINFER_DISPATCH_DTYPE(dtype, {
+      gate_kernel<S><<<grid, 256, 0, stream>>>((S*)x + t0 * ld_x, ld_x, (const S*)g + t0 * ld_g, ld_g, n, act);
+    });
+  }
+  return launch_status();
+}
+
+// out[t, i] = act(in[t, i]) for i < n (in place allowed). act: 0 silu, 1 relu squared, 2 gelu (tanh form), 3 gelu
+// (error function), 4 logistic.
 extern "C" int dinfer_act(int dtype, int act, const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t tokens,
                           int64_t n, hipStream_t stream) {
   if (tokens <= 0 || n <= 0) return OK;
-  if (act < 0 || act > 2) return ERR_UNSUPPORTED;
+  if (act < 0 || act > 4) return ERR_UNSUPPORTED;
   if (ld_in < n || ld_out < n) return ERR_BAD_SHAPE;
   for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
     const int64_t nt = tokens - t0 < 65535 ? tokens - t0 : 65535;

@@ -20,7 +20,7 @@
 //                token the `top` largest (lowest index first among equals), the softmax over the chosen and the shared
 //                expert's sigmoid gate
 //   moe_scatter  counts, offsets, the sorted list and the work list, one workgroup (LDS counters)
-//   moe_combine  out[t] = sum_c share[t, c] * y[t * top + c] + shared_gate[t] * shared[t]
+//   moe_combine  out[t] = sum_c share[t, c] * y[t * top + c] + shared_gate[t] * shared[t]   (no gate: + shared[t])
 #include "common.cuh"
 
 using namespace dinfer;
@@ -40,10 +40,16 @@ struct Groups {
   const void* gate; int64_t ld_gate;   // heads: optional
   int gate_n;               // GATED: rows of each half of W_g
   int tm;                   // rows of a tile: 64 on the vector ALUs, 16 or 128 on the matrix cores
+  int act;                  // not GATED: 0 nothing, 1 silu, 2 gelu (error function) on every result
 };
 
 __device__ __forceinline__ float silu(float x) { return x / (1.f + expf(-x)); }
 __device__ __forceinline__ float sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float plain_act(float x, int act) {
+  if (act == 1) return silu(x);
+  if (act == 2) return 0.5f * x * (1.f + erff(x * 0.7071067811865476f));
+  return x;
+}
 
 constexpr int BM = 64, BN = 64, BK = 16;
 
@@ -140,7 +146,7 @@ __global__ void __launch_bounds__(256) grouped_valu_kernel(Groups p) {
     for (int j = 0; j < 4; ++j) {
       const int gn = n0 + tx * 4 + j;
       if (gn < p.N) {
-        float v = GATED ? silu(acc[i][j]) * acu[i][j] : acc[i][j];
+        float v = GATED ? silu(acc[i][j]) * acu[i][j] : plain_act(acc[i][j], p.act);
         C[cr * p.ldc + gn] = from_f32<O>(v * g);
       }
     }
@@ -252,7 +258,7 @@ __global__ void __launch_bounds__(256) grouped_mfma_big_kernel(Groups p) {
       for (int j = 0; j < (GATED ? 2 : 4); ++j) {
         const int gn = GATED ? n0 + wn * 32 + j * 16 + lr : n0 + wn * 64 + j * 16 + lr;
         if (gn < p.N) {
-          const float v = GATED ? silu(acc[i][j][r]) * acc[i][j + 2][r] : acc[i][j][r];
+          const float v = GATED ? silu(acc[i][j][r]) * acc[i][j + 2][r] : plain_act(acc[i][j][r], p.act);
           C[cr * p.ldc + gn] = from_f32<O>(v * g);
         }
       }
@@ -317,7 +323,7 @@ __global__ void __launch_bounds__(256) grouped_mfma_small_kernel(Groups p) {
   float g = 1.f;
   if (p.gate) g = sigmoid((float)((const bf16*)p.gate)[cr * p.ld_gate + tl.z]);
   O* C = (O*)p.C + (experts ? 0 : (int64_t)tl.z * p.c_zs);
-  C[cr * p.ldc + n0 + col] = from_f32<O>((GATED ? silu(v) * u : v) * g);
+  C[cr * p.ldc + n0 + col] = from_f32<O>((GATED ? silu(v) * u : plain_act(v, p.act)) * g);
 }
 
 // ---- routing ---------------------------------------------------------------------------------------------------
@@ -437,7 +443,7 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const S* __restrict__ 
                                                           const float* __restrict__ shared_gate, S* __restrict__ out,
                                                           int64_t ld_o, int width) {
   const int64_t t = blockIdx.x;
-  const float sg = shared ? shared_gate[t] : 0.f;
+  const float sg = shared ? (shared_gate ? shared_gate[t] : 1.f) : 0.f;   // no gate: the shared output as it is
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float acc = 0.f;
     for (int c = 0; c < top; ++c) acc = fmaf(share[t * top + c], to_f32(y[(t * top + c) * ld_y + i]), acc);
@@ -459,7 +465,7 @@ __global__ void __launch_bounds__(256) moe_combine_bf16x8_kernel(const bf16* __r
                                                                  const float* __restrict__ shared_gate,
                                                                  bf16* __restrict__ out, int64_t ld_o, int width) {
   const int64_t t = blockIdx.x;
-  const float sg = shared ? shared_gate[t] : 0.f;
+  const float sg = shared ? (shared_gate ? shared_gate[t] : 1.f) : 0.f;   // no gate: the shared output as it is
   for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
     float acc[8];
 #pragma unroll
@@ -519,7 +525,8 @@ extern "C" int dinfer_heads_nt(int dtype, const void* A, int64_t lda, int64_t a_
 }
 
 // The products of the experts (see the head of the file). W [experts][rows][ldw] with w_zs elements an expert;
-// gated != 0: rows = 2 N (gate rows, then up rows). max_tiles: the length of `tiles`.
+// gated 1: rows = 2 N (gate rows, then up rows); 0: plain; 2, 3: plain with silu or gelu (error function) on every
+// result. max_tiles: the length of `tiles`.
 extern "C" int dinfer_experts_nt(int dtype, int gated, const void* A, int64_t lda, const void* W, int64_t ldw,
                                  int64_t w_zs, void* C, int64_t ldc, int64_t N, int64_t K, const int32_t* tiles,
                                  int64_t max_tiles, int tile_rows, const int32_t* offsets, const int32_t* perm, int a_div,
@@ -532,8 +539,10 @@ extern "C" int dinfer_experts_nt(int dtype, int gated, const void* A, int64_t ld
   p.A = A; p.lda = lda; p.W = W; p.ldw = ldw; p.w_zs = w_zs; p.C = C; p.ldc = ldc;
   p.N = (int)N; p.K = (int)K; p.tiles = tiles; p.offsets = offsets; p.perm = perm; p.a_div = a_div;
   p.c_to_perm = c_to_perm; p.gate_n = (int)N; p.tm = tile_rows;
+  if (gated < 0 || gated > 3) return ERR_UNSUPPORTED;
+  p.act = gated >= 2 ? gated - 1 : 0;
   if (!mfma_fits(dtype, p) && tile_rows > BM) return ERR_UNSUPPORTED;
-  return gated ? launch_groups<true>(dtype, p, (unsigned)max_tiles, 1, stream)
+  return gated == 1 ? launch_groups<true>(dtype, p, (unsigned)max_tiles, 1, stream)
                : launch_groups<false>(dtype, p, (unsigned)max_tiles, 1, stream);
 }
 

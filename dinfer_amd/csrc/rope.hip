@@ -44,7 +44,8 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
     S* __restrict__ qkv, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, const void* __restrict__ wq,
     const void* __restrict__ wk, int wf32, float eps, float w_offset, const int32_t* __restrict__ pos,
     const float* __restrict__ cos_sin, int rot, int style, S* __restrict__ k_cache, S* __restrict__ v_cache,
-    const int64_t* __restrict__ slots, int H, int Hkv, int D, int page, int Dv) {
+    const int64_t* __restrict__ slots, int H, int Hkv, int D, int page, int Dv, const float* __restrict__ bias,
+    float temp_coef, int temp_every) {
   __shared__ float xs[WAVES][MAX_D];
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -62,7 +63,12 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
     const int hk = item - H - Hkv;
     const S* vs = row + v_off + (int64_t)hk * Dv;
     S* vd = v_cache + ((blk * Hkv + hk) * (int64_t)Dv) * page + off;
-    for (int d = lane; d < Dv; d += 64) vd[(int64_t)d * page] = vs[d];
+    if (bias) {
+      const float* vb = bias + (int64_t)(H + Hkv) * D + (int64_t)hk * Dv;
+      for (int d = lane; d < Dv; d += 64) vd[(int64_t)d * page] = from_f32<S>(to_f32(vs[d]) + vb[d]);
+    } else {
+      for (int d = lane; d < Dv; d += 64) vd[(int64_t)d * page] = vs[d];
+    }
   }
 
   const int hk = item - H;
@@ -72,14 +78,18 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
 
   if (is_qk) {
     float ss = 0.f;
+    const float* hb = bias ? bias + (int64_t)item * D : nullptr;   // q heads, then k heads
     for (int d = lane; d < D; d += 64) {
-      const float v = to_f32(base[d]);
+      float v = to_f32(base[d]);
+      if (hb) v += hb[d];
       x[d] = v;
       ss += v * v;
     }
     if (w) {
       ss = wave_sum(ss);
-      const float inv = 1.f / sqrtf(ss / (float)D + eps);
+      float inv = 1.f / sqrtf(ss / (float)D + eps);
+      // a query grows with its position: 1 + coef ln(floor((p + 1) / every) + 1)
+      if (is_q && temp_every > 0) inv *= 1.f + temp_coef * logf((float)((pos[t] + 1) / temp_every) + 1.f);
       // each lane rescales only the entries it wrote itself
       for (int d = lane; d < D; d += 64) x[d] = x[d] * inv * (ld_param<S>(w, d, wf32) + w_offset);
     }
@@ -391,7 +401,9 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
                                float w_offset, const int32_t* positions, const float* cos_sin, int rotary_dim,
                                int style, void* k_cache, void* v_cache, const int64_t* slot_mapping, int heads,
                                int kv_heads, int head_dim, int page_size, int token_runs, int v_dim,
-                               hipStream_t stream) {
+                               const float* bias, float temp_coef, int temp_every, hipStream_t stream) {
+  // bias (may be null): float [q heads | k heads | v heads], added to the product's output before anything else.
+  // temp_every > 0: q is multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1) with the norm (gains needed).
   // v_dim: the size of a value head, 0 for head_dim. v_cache may be null beside a k_cache (values are not stored).
   if (v_dim <= 0) v_dim = head_dim;
   // token_runs: the tokens come in runs of consecutive positions of a request (prompt portions), so
@@ -404,8 +416,9 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   if ((q_gain == nullptr) != (k_gain == nullptr)) return ERR_BAD_SHAPE;
   const int items = heads + 2 * kv_heads;
   const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES - 1) / WAVES));
+  if (temp_every > 0 && !q_gain) return ERR_UNSUPPORTED;
   const bool whole_head_neox = style == 0 && head_dim % 8 == 0 && (!cos_sin || rotary_dim == head_dim) &&
-                               v_dim == head_dim && (v_cache || !slot_mapping);
+                               v_dim == head_dim && (v_cache || !slot_mapping) && !bias && temp_every <= 0;
   const bool vec_ok = dtype == DT_BF16 && (head_dim == 64 || head_dim == 128 || head_dim == 256) && ld % 8 == 0 &&
                       q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
                       ((uintptr_t)q_gain % 16) == 0 && ((uintptr_t)k_gain % 16) == 0 && ((uintptr_t)cos_sin % 16) == 0 &&
@@ -451,7 +464,7 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
     qkv_post_kernel<S><<<grid, WAVES * 64, 0, stream>>>((S*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps,
                                                         w_offset, positions, cos_sin, rotary_dim, style, (S*)k_cache,
                                                         (S*)v_cache, slot_mapping, heads, kv_heads, head_dim,
-                                                        page_size, v_dim);
+                                                        page_size, v_dim, bias, temp_coef, temp_every);
   });
   return launch_status();
 }

@@ -40,7 +40,8 @@ SIGNATURES = {
     "dinfer_rmsnorm": ("norm", [_I, _P, _P, _P, _P, _I, _P, _L, _L, _L, _L, _F, _F, _P]),
     "dinfer_qkv_post": (
         "rope",
-        [_I, _P, _L, _L, _L, _L, _L, _P, _P, _I, _F, _F, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+        [_I, _P, _L, _L, _L, _L, _L, _P, _P, _I, _F, _F, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I,
+         _P],
     ),
     "dinfer_attn_paged_ref": (
         "attention_ref",
@@ -58,6 +59,15 @@ SIGNATURES = {
     "dinfer_delta_conv_update": ("delta", [_I, _P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _P]),
     "dinfer_delta_recurrence": ("delta", [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P]),
     "dinfer_delta_out": ("delta", [_I, _P, _L, _P, _L, _L, _P, _P, _L, _L, _L, _I, _I, _F, _F, _P]),
+    "dinfer_gate": ("elementwise", [_I, _I, _P, _L, _P, _L, _L, _L, _P]),
+    "dinfer_rot_widen": ("decay", [_I, _P, _L, _L, _L, _L, _P, _P, _I, _F, _P, _L, _L, _I, _I, _I, _P]),
+    "dinfer_conv_silu": ("decay", [_I, _P, _L, _L, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _L, _I, _I, _I, _P]),
+    "dinfer_decay_recurrence": ("decay", [_P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I,
+                                          _I, _P]),
+    "dinfer_gated_group_norm": ("decay", [_I, _P, _L, _P, _L, _P, _I, _P, _L, _L, _P, _P, _L, _L, _L, _I, _I, _F, _F, _I,
+                                          _P]),
+    "dinfer_streams_expand": ("streams", [_I, _P, _L, _P, _L, _L, _I, _I, _P]),
+    "dinfer_streams_step": ("streams", [_I, _P, _L, _I, _I, _P, _P, _L, _P, _P, _P, _P, _P, _F, _P, _L, _P, _L, _L, _P]),
     "dinfer_attn_mfma_supports": ("attention", [_I, _I, _I, _I]),
     "dinfer_attn_flash": (
         "attention",

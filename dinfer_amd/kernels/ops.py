@@ -154,7 +154,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float
     return out
 
 
-ACTS = {"silu": 0, "relu2": 1, "gelu_tanh": 2}   # activations of one argument -> their code in the C interface
+# activations of one argument -> their code in the C interface ("gelu": with the error function)
+ACTS = {"silu": 0, "relu2": 1, "gelu_tanh": 2, "gelu": 3, "sigmoid": 4}
 
 
 def act(x: torch.Tensor, out: torch.Tensor, tokens: int, kind: str) -> torch.Tensor:
@@ -167,6 +168,18 @@ def act(x: torch.Tensor, out: torch.Tensor, tokens: int, kind: str) -> torch.Ten
     lib.call("dinfer_act", dtype_code(x.dtype), ACTS[kind], x.data_ptr(), _rows(x), out.data_ptr(), _rows(out), tokens, n,
              _stream())
     return out
+
+
+def gate(x: torch.Tensor, g: torch.Tensor, tokens: int, kind: str) -> torch.Tensor:
+    """x[t, i] *= act(g[t, i]) in place; x and g are views of equally many columns (blocks of wider buffers)."""
+    _need_gpu(x, g)
+    if kind not in ACTS:
+        raise lib.KernelError(f"activation {kind!r} has no kernel (known: {sorted(ACTS)})")
+    n = x.shape[1]
+    assert g.shape[1] == n and x.dtype == g.dtype and x.shape[0] >= tokens and g.shape[0] >= tokens
+    lib.call("dinfer_gate", dtype_code(x.dtype), ACTS[kind], x.data_ptr(), _rows(x), g.data_ptr(), _rows(g), tokens, n,
+             _stream())
+    return x
 
 
 def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, eps: float,
@@ -327,6 +340,145 @@ def delta_out(o: torch.Tensor, proj: torch.Tensor, g_off: int, weight: torch.Ten
     return out
 
 
+# ---- recurrences with a scalar decay ---------------------------------------------------------------
+DECAY_MAX_DIM = 256      # the largest key size of the recurrence kernel
+
+
+def rot_widen(proj: torch.Tensor, tokens: int, *, q_off: int, k_off: int, v_off: int, positions: torch.Tensor,
+              cos_sin: torch.Tensor | None, rotary_dim: int, k_scale: float, work: torch.Tensor, heads: int, dim: int,
+              vdim: int) -> torch.Tensor:
+    """work[t] = rotated q (heads dim) | rotated k * k_scale | v (heads vdim), float32; the first rotary_dim entries
+    of a head turn in pairs (i, i + rotary_dim / 2) by the table row [cos | sin] of the token's position."""
+    _need_gpu(proj, positions, cos_sin, work)
+    assert work.dtype == torch.float32 and work.shape[0] >= tokens and work.shape[1] >= heads * (2 * dim + vdim)
+    assert proj.shape[0] >= tokens and max(q_off + heads * dim, k_off + heads * dim, v_off + heads * vdim) <= proj.shape[1]
+    assert positions.dtype == torch.int32 and positions.numel() >= tokens
+    if cos_sin is not None:
+        assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rotary_dim
+    lib.call("dinfer_rot_widen", dtype_code(proj.dtype), proj.data_ptr(), _rows(proj), q_off, k_off, v_off,
+             positions.data_ptr(), _ptr(cos_sin), rotary_dim if cos_sin is not None else 0, float(k_scale), work.data_ptr(),
+             _rows(work), tokens, heads, dim, vdim, _stream())
+    return work
+
+
+def conv_silu(proj: torch.Tensor, tokens: int, *, x_off: int, dt_off: int, taps: torch.Tensor, bias: torch.Tensor | None,
+              a_log: torch.Tensor, dt_bias: torch.Tensor, conv_state: torch.Tensor | None, state_slots: torch.Tensor,
+              cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, work: torch.Tensor, num_reqs: int) -> torch.Tensor:
+    """Short causal convolution with bias over the step's rows and the request's stored inputs, then silu, for the
+    C = taps.shape[0] channels from column x_off; step sizes dt = softplus(proj[dt_off + h] + dt_bias[h]) and decays
+    exp(-exp(a_log[h]) dt). work [T, >= C + 2 H] float32: channels | dt | decay."""
+    _need_gpu(proj, taps, bias, a_log, dt_bias, conv_state, state_slots, cu_seqlens, seq_lens, work)
+    C, K = taps.shape
+    H = a_log.numel()
+    assert taps.dtype == torch.float32 and taps.is_contiguous() and a_log.dtype == dt_bias.dtype == torch.float32
+    assert dt_bias.numel() == H and (bias is None or (bias.dtype == torch.float32 and bias.numel() == C))
+    assert work.dtype == torch.float32 and work.shape[0] >= tokens and work.shape[1] >= C + 2 * H
+    assert proj.shape[0] >= tokens and max(x_off + C, dt_off + H) <= proj.shape[1]
+    if K > 1:
+        assert conv_state is not None and conv_state.dtype == proj.dtype and conv_state.is_contiguous()
+        assert tuple(conv_state.shape[1:]) == (C, K - 1)
+    lib.call("dinfer_conv_silu", dtype_code(proj.dtype), proj.data_ptr(), _rows(proj), x_off, dt_off, taps.data_ptr(),
+             _ptr(bias), a_log.data_ptr(), dt_bias.data_ptr(), _ptr(conv_state) if K > 1 else None, state_slots.data_ptr(),
+             cu_seqlens.data_ptr(), seq_lens.data_ptr(), work.data_ptr(), _rows(work), num_reqs, tokens, C, H, K, _stream())
+    return work
+
+
+def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, gain: torch.Tensor | None,
+                     state: torch.Tensor, out: torch.Tensor, *, state_slots: torch.Tensor, cu_seqlens: torch.Tensor,
+                     seq_lens: torch.Tensor, num_reqs: int, groups: int, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """Per request and head, token by token: S <- decay S + gain k v^T, out = S^T q. q, k: float32 views [T, groups dim]
+    (head h reads group h // (heads / groups)); v [T, heads vdim]; decay [T, heads], or [heads] for one decay a head;
+    gain [T, heads] or None. state [slots, heads, vdim, dim] float32, updated in place; out [T, >= heads vdim] float32."""
+    _need_gpu(q, k, v, decay, gain, state, out, state_slots, cu_seqlens, seq_lens)
+    tensors = [q, k, v, decay, state, out] + ([gain] if gain is not None else [])
+    assert all(t.dtype == torch.float32 for t in tensors) and state.is_contiguous()
+    assert tuple(state.shape[1:]) == (heads, vdim, dim) and out.shape[1] >= heads * vdim
+    assert q.shape[1] >= groups * dim and k.shape[1] >= groups * dim and v.shape[1] >= heads * vdim
+    if decay.dim() == 1:
+        assert decay.numel() == heads and decay.is_contiguous()
+        ldd = 0
+    else:
+        assert decay.shape[1] >= heads
+        ldd = _rows(decay)
+    assert gain is None or gain.shape[1] >= heads
+    lib.call("dinfer_decay_recurrence", q.data_ptr(), _rows(q), k.data_ptr(), _rows(k), v.data_ptr(), _rows(v),
+             decay.data_ptr(), ldd, _ptr(gain), _rows(gain) if gain is not None else 0, state.data_ptr(),
+             state_slots.data_ptr(), cu_seqlens.data_ptr(), seq_lens.data_ptr(), out.data_ptr(), _rows(out), num_reqs,
+             groups, heads, dim, vdim, _stream())
+    return out
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, z_off: int, out: torch.Tensor, tokens: int, *, groups: int,
+                     group: int, eps: float, weight: torch.Tensor | None = None, x: torch.Tensor | None = None,
+                     skip: torch.Tensor | None = None, vdim: int = 0, col_off: int = 0, out_scale: float = 1.0,
+                     gate_first: bool = True) -> torch.Tensor:
+    """u = (y + skip[c // vdim] x) * silu(z[:, z_off + c]); out[:, col_off + c] = u / rms over c's group of `group`
+    columns (eps inside the root) * weight[c] * out_scale. gate_first False: the gate multiplies after the norm
+    instead. y, x float32; z and out in the activations' type."""
+    _need_gpu(y, z, out, weight, x, skip)
+    n = groups * group
+    assert y.dtype == torch.float32 and y.shape[1] >= n and z.dtype == out.dtype
+    assert min(y.shape[0], z.shape[0], out.shape[0]) >= tokens and z_off + n <= z.shape[1] and col_off + n <= out.shape[1]
+    assert weight is None or (weight.dtype == torch.float32 and weight.numel() == n and weight.is_contiguous())
+    if skip is not None:
+        assert x is not None and x.dtype == torch.float32 and x.shape[1] >= n and x.shape[0] >= tokens
+        assert skip.dtype == torch.float32 and vdim > 0 and skip.numel() * vdim == n
+    lib.call("dinfer_gated_group_norm", dtype_code(out.dtype), y.data_ptr(), _rows(y), _ptr(x) if skip is not None else None,
+             _rows(x) if skip is not None else 0, _ptr(skip), int(vdim), z.data_ptr(), _rows(z), z_off, _ptr(weight),
+             out.data_ptr(), _rows(out), col_off, tokens, groups, group, float(eps), float(out_scale), 1 if gate_first else 0, _stream())
+    return out
+
+
+# ---- several residual streams ----------------------------------------------------------------------
+STREAMS_MAX = 8          # streams a token the kernel holds in registers
+STREAMS_MAX_WIDTH = 12288
+
+
+def streams_expand(src: torch.Tensor, x: torch.Tensor, tokens: int, n: int) -> torch.Tensor:
+    """x[t, s W + c] = src[t, c] for every stream s < n; x float32 [T, n W]."""
+    _need_gpu(src, x)
+    W = src.shape[1]
+    assert x.dtype == torch.float32 and x.shape[1] == n * W and min(src.shape[0], x.shape[0]) >= tokens
+    lib.call("dinfer_streams_expand", dtype_code(src.dtype), src.data_ptr(), _rows(src), x.data_ptr(), _rows(x), tokens, n,
+             W, _stream())
+    return x
+
+
+def streams_step(x: torch.Tensor, n_rows: int, n: int, *, dtype: torch.dtype, branch: torch.Tensor | None = None,
+                 mix: torch.Tensor | None = None, out_weights: torch.Tensor | None = None,
+                 read: torch.Tensor | None = None, gain: torch.Tensor | None = None, bias: torch.Tensor | None = None,
+                 eps: float = 0.0, out: torch.Tensor | None = None, u_out: torch.Tensor | None = None,
+                 rows: torch.Tensor | None = None):
+    """One pass over the rows of x (float32 [T, n W], n streams side by side): with a branch y [T, W],
+    x_t <- sum_s mix[s, t] x_s + out_weights[t] y for all streams at once; with `read`, u = sum_s read[s] x_s, which goes
+    to u_out (float32) as it is, or, with gain (and bias), through a layer norm to out (in `dtype`, the type of branch
+    and out). rows: int32 source rows; then the streams themselves stay as they are."""
+    _need_gpu(x, branch, mix, out_weights, read, gain, bias, out, u_out, rows)
+    W = x.shape[1] // n
+    assert x.dtype == torch.float32 and x.shape[1] == n * W
+    small = [t for t in (mix, out_weights, read, gain, bias) if t is not None]
+    assert all(t.dtype == torch.float32 and t.is_contiguous() for t in small)
+    if branch is not None:
+        assert branch.dtype == dtype and branch.shape[1] == W and mix.numel() == n * n and out_weights.numel() == n
+        assert rows is not None or branch.shape[0] >= n_rows
+    if read is not None:
+        assert read.numel() == n
+        if gain is not None:
+            assert gain.numel() == W and (bias is None or bias.numel() == W)
+            assert out is not None and out.dtype == dtype and out.shape[1] == W and out.shape[0] >= n_rows
+        else:
+            assert u_out is not None and u_out.dtype == torch.float32 and u_out.shape[1] == W and u_out.shape[0] >= n_rows
+    if rows is not None:
+        assert rows.dtype == torch.int32 and rows.is_contiguous() and rows.numel() >= n_rows
+    else:
+        assert x.shape[0] >= n_rows
+    lib.call("dinfer_streams_step", dtype_code(dtype), x.data_ptr(), _rows(x), n, W, _ptr(rows), _ptr(branch),
+             _rows(branch) if branch is not None else 0, _ptr(mix), _ptr(out_weights), _ptr(read), _ptr(gain), _ptr(bias),
+             float(eps), _ptr(out), _rows(out) if out is not None else 0, _ptr(u_out),
+             _rows(u_out) if u_out is not None else 0, n_rows, _stream())
+    return out if gain is not None else u_out
+
+
 # ---- latent attention ----------------------------------------------------------------------------
 # Cache pages [blocks, page, R + dr]: one row a token, the normed latent and then the rotated shared key part.
 LATENT_MAX_RANK = 1024   # the largest latent the attention kernels hold in registers
@@ -438,6 +590,9 @@ MOE_MAX_EXPERTS = 1024   # the routing and sorting kernels keep one number an ex
 MOE_MAX_TOP = 64         # a lane of the routing wave keeps one choice
 
 
+EXPERT_ACTS = {"silu": 2, "gelu": 3}    # activations the plain (not gated) expert products apply -> their code
+
+
 def moe_tile_rows(dtype: torch.dtype, entries: int, experts: int, k_in: int, k_mid: int) -> int:
     """Rows of a row tile for the two products of a routed layer over `entries` (token, choice) pairs: what the kernel
     that will run them takes (16 where an expert gets few rows, 128 for many, 64 on the vector ALUs)."""
@@ -462,7 +617,7 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, shared_gate_w: torch.Tensor
     assert z.dtype == torch.float32 and z.is_contiguous() and z.numel() >= tokens * (experts + 1)
     if shared_gate_w is not None:
         assert shared_gate_w.dtype == torch.float32 and shared_gate_w.numel() == width and shared_gate_w.is_contiguous()
-        assert shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens
+        assert shared_gate is None or (shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens)
     lib.call("dinfer_moe_route", dtype_code(x.dtype), x.data_ptr(), _rows(x), tokens, router.data_ptr(),
              _ptr(shared_gate_w), experts, top, width, z.data_ptr(), idx.data_ptr(), share.data_ptr(),
              _ptr(shared_gate) if shared_gate_w is not None else 0, _stream())
@@ -484,17 +639,19 @@ def moe_scatter(idx: torch.Tensor, entries: int, experts: int, offsets: torch.Te
 
 def experts_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, entries: int, tiles: torch.Tensor,
                offsets: torch.Tensor, perm: torch.Tensor, *, gated: bool, a_div: int, c_to_perm: bool,
-               tile_rows: int) -> torch.Tensor:
+               tile_rows: int, act: str | None = None) -> torch.Tensor:
     """The products of all experts in one launch. w [experts, rows, K]; gated: rows = 2 N, gate rows first, and
     out = silu(a Wg^T) * (a Wu^T). a_div > 0: the row of sorted place i is a[perm[i] // a_div] (the step's tokens),
     0: a[i]. c_to_perm: the result of sorted place i goes to out[perm[i]], else to out[i]. tile_rows: what moe_scatter
-    made the work list with."""
+    made the work list with. act (not gated): "silu" or "gelu" (error function) on every result."""
     _need_gpu(a, w, out, tiles, offsets, perm)
+    if act is not None and (gated or act not in EXPERT_ACTS):
+        raise lib.KernelError(f"experts: activation {act!r} has no kernel here (known: {sorted(EXPERT_ACTS)}, not gated)")
     experts, rows, k = w.shape
     n = rows // 2 if gated else rows
     assert w.is_contiguous() and a.dtype == w.dtype == out.dtype and a.shape[1] == k and out.shape[1] == n
     assert out.shape[0] >= entries and (a_div > 0 or a.shape[0] >= entries)
-    lib.call("dinfer_experts_nt", dtype_code(a.dtype), 1 if gated else 0, a.data_ptr(), _rows(a), w.data_ptr(), k,
+    lib.call("dinfer_experts_nt", dtype_code(a.dtype), 1 if gated else EXPERT_ACTS[act] if act else 0, a.data_ptr(), _rows(a), w.data_ptr(), k,
              rows * k, out.data_ptr(), _rows(out), n, k, tiles.data_ptr(), moe_max_tiles(entries, experts, tile_rows),
              int(tile_rows), offsets.data_ptr(), perm.data_ptr(), int(a_div), 1 if c_to_perm else 0, _stream())
     return out
@@ -502,14 +659,14 @@ def experts_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, entries: int
 
 def moe_combine(y: torch.Tensor, share: torch.Tensor, top: int, shared: torch.Tensor | None,
                 shared_gate: torch.Tensor | None, out: torch.Tensor, tokens: int) -> torch.Tensor:
-    """out[t] = sum_c share[t, c] * y[t * top + c] (+ shared_gate[t] * shared[t])."""
+    """out[t] = sum_c share[t, c] * y[t * top + c] (+ shared_gate[t] * shared[t], or + shared[t] without a gate)."""
     _need_gpu(y, share, shared, shared_gate, out)
     width = out.shape[1]
     assert y.shape[1] == width and y.dtype == out.dtype and y.shape[0] >= tokens * top and out.shape[0] >= tokens
     assert share.dtype == torch.float32 and share.numel() >= tokens * top
     if shared is not None:
         assert shared.dtype == out.dtype and shared.shape[1] == width and shared.shape[0] >= tokens
-        assert shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens
+        assert shared_gate is None or (shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens)
     lib.call("dinfer_moe_combine", dtype_code(y.dtype), y.data_ptr(), _rows(y), share.data_ptr(), top, _ptr(shared),
              _rows(shared) if shared is not None else 0, _ptr(shared_gate), out.data_ptr(), _rows(out), tokens, width,
              _stream())
@@ -556,8 +713,11 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
              v_off: int, q_gain: torch.Tensor | None, k_gain: torch.Tensor | None, eps: float, gain_offset: float,
              positions: torch.Tensor, cos_sin: torch.Tensor | None, rotary_dim: int, rope_style: int,
              k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, slot_mapping: torch.Tensor | None,
-             page_size: int, token_runs: bool = True, v_dim: int | None = None) -> None:
+             page_size: int, token_runs: bool = True, v_dim: int | None = None, bias: torch.Tensor | None = None,
+             q_temp: tuple | None = None) -> None:
     """Per-head q/k norm, rotation, q written back in place, k and v written to the cache pages.
+    bias: float32 [q heads | k heads | v heads], added to the product's output first. q_temp (coef, every): q is
+    multiplied by 1 + coef ln(floor((p + 1) / every) + 1) at position p, together with the norm.
     v_dim: the size of a value head where it is not head_dim. v_cache None beside a k_cache: the values are not stored
     (a layer whose values are its keys reads them from the key pages).
 
@@ -578,6 +738,11 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
         assert _is_param_f32(k_gain, qkv.dtype) == wf32
     if cos_sin is not None:
         assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rotary_dim
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous()
+        assert bias.numel() == (heads + kv_heads) * head_dim + kv_heads * vd
+    if q_temp is not None:
+        assert q_gain is not None and int(q_temp[1]) > 0
     if slot_mapping is not None:
         assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() >= tokens
         assert k_cache is not None
@@ -586,7 +751,8 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
     lib.call("dinfer_qkv_post", dtype_code(qkv.dtype), qkv.data_ptr(), tokens, ld, q_off, k_off, v_off,
              _ptr(q_gain), _ptr(k_gain), wf32, float(eps), float(gain_offset), positions.data_ptr(), _ptr(cos_sin),
              rotary_dim, rope_style, _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), heads, kv_heads, head_dim,
-             page_size, int(token_runs), vd, _stream())
+             page_size, int(token_runs), vd, _ptr(bias), float(q_temp[0]) if q_temp else 0.0,
+             int(q_temp[1]) if q_temp else 0, _stream())
 
 
 def attn_paged_ext(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor | None,

@@ -9,8 +9,13 @@ Options, each a constructor parameter that is off by default: values of a size o
 `keep_first` keys staying visible behind the window; a learned sink a head in the softmax's denominator (`sink`, a
 tensor [heads]); a bias that takes 2^(-slope_exp (h + 1) / heads) times the distance off the scores (`slope_exp`);
 values that are the keys (`values_are_keys`: no value projection, no value pages); the output multiplied by
-`out_scale`; tensor names (`names`). A layer that uses any of the first five runs the plain kernel with options
-(csrc/attention_ref.hip) for prompt portions and single rows alike; the matrix-core kernels serve the others.
+`out_scale`; tensor names (`names`). Further: biases on the q, k and v projections (`bias`); q and k divided by their
+root mean square a head without a gain (`qk_unit_eps`); a query that grows with its position, times
+1 + coef ln(floor((p + 1) / every) + 1) (`q_temp = (coef, every)`); a sink of a fixed score instead of a learned one
+(`sink_value`: 0.0 adds one to the softmax's denominator); the concatenated heads multiplied by an activation of one
+more projection of the mixer's input before the output projection (`gate`: "sigmoid" or "silu"). A layer that uses any
+option runs the flash kernel with options on the matrix cores where its sizes allow, else the plain kernel with options
+(csrc/attention_ref.hip), for prompt portions and single rows alike; the matrix-core kernels serve the others.
 """
 from __future__ import annotations
 
@@ -31,12 +36,15 @@ class Attention(Mixer):
     capturable_portions = True   # the choice of kernels follows the step's counts alone
 
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-             "q_norm": "q_norm.", "k_norm": "k_norm.", "sink": "sinks"}
+             "q_norm": "q_norm.", "k_norm": "k_norm.", "sink": "sinks", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias",
+             "v_bias": "v_proj.bias", "g": "g_proj.weight"}
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position: PartSpec,
                  qk_norm: PartSpec | None = None, window: int | None = None, scale: float | None = None,
                  v_dim: int | None = None, keep_first: int = 0, sink: bool = False, slope_exp: float = 0.0,
-                 values_are_keys: bool = False, out_scale: float = 1.0, names: dict | None = None):
+                 values_are_keys: bool = False, out_scale: float = 1.0, names: dict | None = None, bias: bool = False,
+                 qk_unit_eps: float | None = None, q_temp: tuple | None = None, sink_value: float | None = None,
+                 gate: str | None = None):
         if heads % kv_heads:
             raise ValueError(f"heads {heads} not divisible by kv_heads {kv_heads}")
         if head_dim <= 0 or head_dim > ops.MAX_HEAD_DIM:   # said at build, not at the first step
@@ -54,12 +62,29 @@ class Attention(Mixer):
         if self.keep_first and not window:
             self.keep_first = 0     # without a window every key stays visible anyway
         self.names = dict(self.NAMES, **(names or {}))
+        self.bias, self.qk_unit_eps, self.gate = bool(bias), qk_unit_eps, gate
+        self.q_temp = None if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
+        self.sink_value = None if sink_value is None else float(sink_value)
+        if self.sink and self.sink_value is not None:
+            raise ValueError("attention: a sink is learned (`sink`) or of a fixed score (`sink_value`), not both")
+        if qk_unit_eps is not None and qk_norm is not None:
+            raise ValueError("attention: q and k are normed with gains (`qk_norm`) or without (`qk_unit_eps`), not both")
+        if self.q_temp is not None and (self.q_temp[1] <= 0 or (qk_norm is None and qk_unit_eps is None)):
+            raise ValueError("attention: a query temperature needs every > 0 and a per-head norm of q (it rides in it)")
+        if gate is not None and gate not in ("sigmoid", "silu"):
+            raise ValueError(f"attention: gate {gate!r} unknown (known: 'sigmoid', 'silu')")
+        if self.bias and self.values_are_keys:
+            raise ValueError("attention: biases with values that are the keys are not built")
         # what the matrix-core kernels do not do runs through the plain kernel with options
         self.extended = bool(self.v_dim != head_dim or self.keep_first or self.sink or self.slope_exp
-                             or self.values_are_keys or self.out_scale != 1.0)
+                             or self.values_are_keys or self.out_scale != 1.0 or self.bias or qk_unit_eps is not None
+                             or self.q_temp is not None or self.sink_value is not None or gate is not None)
         self.q_size, self.kv_size = heads * head_dim, kv_heads * head_dim
         self.v_size = 0 if self.values_are_keys else kv_heads * self.v_dim
-        self.qkv = Linear(hidden, self.q_size + self.kv_size + self.v_size)
+        self.g_size = heads * self.v_dim if gate is not None else 0
+        self.g_off = self.q_size + self.kv_size + self.v_size
+        self.qkv = Linear(hidden, self.q_size + self.kv_size + self.v_size + self.g_size)
+        self.bias_vec = self.unit_gain = None
         self.o = Linear(heads * self.v_dim, hidden)
         self.sinks = None
         # decided in bind: the matrix-core flash kernel with options serves bfloat16 layers whose values have the keys'
@@ -92,6 +117,12 @@ class Attention(Mixer):
                     t[nm[which] + n] = spec
         if self.sink:
             t[nm["sink"]] = TensorSpec((self.heads,))
+        if self.bias:
+            t[nm["q_bias"]] = TensorSpec((self.q_size,), init="zeros")
+            t[nm["k_bias"]] = TensorSpec((self.kv_size,), init="zeros")
+            t[nm["v_bias"]] = TensorSpec((self.v_size,), init="zeros")
+        if self.gate is not None:
+            t[nm["g"]] = TensorSpec((self.g_size, Hd))
         for n, spec in self.position.tensors().items():   # an encoding with parameters of its own (rotations have none)
             t["position." + n] = spec
         return t
@@ -99,7 +130,7 @@ class Attention(Mixer):
     # ---- the middle part alone, for a mixer that joins several (parts/joined.py) ------------------
     @property
     def in_columns(self) -> int:
-        return self.q_size + self.kv_size + self.v_size
+        return self.q_size + self.kv_size + self.v_size + self.g_size
 
     @property
     def out_columns(self) -> int:
@@ -111,6 +142,8 @@ class Attention(Mixer):
         rows = [get(nm["q"], compute=True), get(nm["k"], compute=True)]
         if not self.values_are_keys:
             rows.append(get(nm["v"], compute=True))
+        if self.gate is not None:
+            rows.append(get(nm["g"], compute=True))
         return torch.cat(rows, dim=0)
 
     def out_weight(self, get) -> torch.Tensor:
@@ -128,6 +161,13 @@ class Attention(Mixer):
             self.k_norm.load(lambda n, **kw: get(nm["k_norm"] + n, **kw))
         if self.sink:
             self.sinks = get(nm["sink"]).float().contiguous()
+        some = get(nm["q"], compute=True)
+        if self.sink_value is not None:
+            self.sinks = torch.full((self.heads,), self.sink_value, dtype=torch.float32, device=some.device)
+        if self.bias:     # small parameters in 32 bits (exact for a bfloat16 file): q heads | k heads | v heads
+            self.bias_vec = torch.cat([get(nm[k]).float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
+        if self.qk_unit_eps is not None:
+            self.unit_gain = torch.ones(self.head_dim, dtype=torch.float32, device=some.device)
         self.position.load(lambda n, **kw: get("position." + n, **kw))
 
     def bind_core(self, ctx):
@@ -140,7 +180,7 @@ class Attention(Mixer):
     def bind(self, ctx):
         ws = ctx.workspace
         self.bind_core(ctx)
-        self.qkv_buf = ws.buffer("qkv", self.q_size + self.kv_size + self.v_size)
+        self.qkv_buf = ws.buffer("qkv", self.qkv.out_features)
         self.attn_buf = ws.buffer("attn", self.heads * self.v_dim)
         self.out_buf = ws.buffer("mixer_out", self.hidden)
         self.attn_ws = attn_kernels.Workspace(ctx, self.heads, self.kv_heads, self.head_dim)
@@ -203,15 +243,23 @@ class Attention(Mixer):
         if not pos.fused:
             raise NotImplementedError("attention with options takes a rotation by a table, or none")
         vd = self.v_dim
+        q_gain, k_gain = (qn.weight, self.k_norm.weight) if qn else (self.unit_gain, self.unit_gain)
+        eps = qn.eps if qn else (self.qk_unit_eps or 0.0)
         ops.qkv_post(qkv_buf, T, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim, q_off=col,
                      k_off=col + self.q_size,     # (values that are the keys: the key columns as the product left them)
                      v_off=col + self.q_size + (0 if self.values_are_keys else self.kv_size),
                      positions=batch.positions, page_size=self.page_size,
-                     q_gain=qn.weight if qn else None, k_gain=self.k_norm.weight if qn else None,
-                     eps=qn.eps if qn else 0.0, gain_offset=qn.weight_offset if qn else 0.0,
+                     q_gain=q_gain, k_gain=k_gain, eps=eps, gain_offset=qn.weight_offset if qn else 0.0,
                      cos_sin=pos.table(), rotary_dim=pos.rotary_dim, rope_style=pos.style,
                      k_cache=cache.k, v_cache=cache.v, slot_mapping=batch.slot_mapping[g] if cache.owner else None,
-                     token_runs=False, v_dim=vd)
+                     token_runs=False, v_dim=vd, bias=self.bias_vec, q_temp=self.q_temp)
+        self._attend_ext(qkv_buf, col, attn_buf, out_col, batch, cache)
+        if self.gate is not None:
+            n = self.heads * vd
+            ops.gate(attn_buf[:, out_col:out_col + n], qkv_buf[:, col + self.g_off:col + self.g_off + n], T, self.gate)
+
+    def _attend_ext(self, qkv_buf, col, attn_buf, out_col, batch, cache: CacheView):
+        T, g, vd = batch.num_tokens, cache.group, self.v_dim
         if self.mfma_ext:
             ops.attn_flash_ext(qkv_buf[:, col:], attn_buf[:, out_col:], cache.k, cache.v, batch.block_table[g],
                                batch.cu_seqlens, batch.seq_lens, batch.num_reqs, batch.max_q_len, scale=self.scale,

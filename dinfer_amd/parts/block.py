@@ -190,3 +190,111 @@ class SandwichBlock(Block):
         if next_norm is None:
             return None
         return Carried(None, None, 0, 0.0, self.hidden, next_norm, hidden, self.normed, T, ready=True)
+
+
+class StreamsWrite:
+    """A sublayer's output that is still to be written into the residual streams (x_t <- sum_s mix[s, t] x_s +
+    out[t] y): left pending by a `streams` block so that the kernel which reads the streams next does the write in the
+    same pass. `settle(rows)` does it alone, for whoever needs the streams whole (the model's end, something added
+    between layers)."""
+    __slots__ = ("streams", "n", "branch", "mix", "out")
+
+    def __init__(self, streams, n, branch, mix, out):
+        self.streams, self.n, self.branch, self.mix, self.out = streams, n, branch, mix, out
+
+    def settle(self, rows: int) -> None:
+        ops.streams_step(self.streams, rows, self.n, dtype=self.branch.dtype, branch=self.branch, mix=self.mix,
+                         out_weights=self.out)
+
+
+@BLOCKS.register("streams")
+class StreamsBlock(Block):
+    """Pre-norm sublayers around `streams` residual streams a token instead of one ("hyper-connections"). For each
+    sublayer (the mixer, then the feed-forward) with its tensors in (streams), mix (streams x streams, [from, to]) and
+    out (streams):
+
+        u = sum_s in[s] x_s;   y = sublayer(norm(u));   x_t <- sum_s mix[s, t] x_s + out[t] y   (all t from the old x)
+
+    `hidden` is [T, streams * width] float32, the streams side by side. One kernel a sublayer boundary does the write
+    of the sublayer before, the read for the next and its norm (a layer norm with gain and bias); the write of a block's
+    last sublayer is left pending for the next block's first kernel. params: streams, the prefixes and names."""
+
+    def __init__(self, hidden: int, layer: LayerSpec, streams: int, mixer_prefix: str = "mix.", ff_prefix: str = "mlp.",
+                 norm_a: str = "norm1", norm_b: str = "norm2", hc_a: str = "hc1.", hc_b: str = "hc2."):
+        if not 0 < streams <= ops.STREAMS_MAX or hidden > ops.STREAMS_MAX_WIDTH:
+            raise ValueError(f"streams block: {streams} streams of width {hidden} have no kernel (up to "
+                             f"{ops.STREAMS_MAX} of {ops.STREAMS_MAX_WIDTH})")
+        self.hidden, self.n = hidden, streams
+        self.mixer = MIXERS.get(layer.mixer.kind)(hidden=hidden, **layer.mixer.params)
+        self.ff = FEED_FORWARDS.get(layer.feed_forward.kind)(hidden=hidden, **layer.feed_forward.params)
+        if getattr(self.ff, "absent", False):
+            self.ff = None
+        ncls = NORMS.get(layer.norm.kind)
+        self.norms = [(norm_a, ncls(hidden, **layer.norm.params))]
+        self.hc_names = [hc_a]
+        if self.ff is not None:
+            self.norms.append((norm_b, ncls(hidden, **layer.norm.params)))
+            self.hc_names.append(hc_b)
+        for _, nm in self.norms:
+            if not hasattr(nm, "has_bias"):
+                raise ValueError("the streams arrangement takes layer norms (gain and optional bias)")
+        self.prefixes = (mixer_prefix, ff_prefix)
+        self.hc = []
+
+    def _parts(self):
+        out = [(self.prefixes[0], self.mixer)] + list(self.norms)
+        if self.ff is not None:
+            out.append((self.prefixes[1], self.ff))
+        return out
+
+    @property
+    def capturable(self):
+        return all(part.capturable for _, part in self._parts())
+
+    @property
+    def capturable_portions(self):
+        return all(part.capturable and part.capturable_portions for _, part in self._parts())
+
+    def tensors(self):
+        from .spec import TensorSpec
+        t = {p + n: s for p, part in self._parts() for n, s in part.tensors().items()}
+        for hc in self.hc_names:
+            t[hc + "in"] = TensorSpec((self.n,), init="ones")
+            t[hc + "out"] = TensorSpec((self.n,), init="ones")
+            t[hc + "mix"] = TensorSpec((self.n, self.n), init="eye")
+        return t
+
+    def load(self, get):
+        for p, part in self._parts():
+            part.load(_sub(get, p))
+        # small parameters in 32 bits (exact for a bfloat16 file): they act on the residual streams
+        self.hc = [tuple(get(hc + k).float().contiguous() for k in ("in", "mix", "out")) for hc in self.hc_names]
+
+    def bind(self, ctx):
+        for _, part in self._parts():
+            part.bind(ctx)
+        self.normed = ctx.workspace.buffer("normed", self.hidden)
+
+    def _boundary(self, hidden, pending, which, T):
+        """The write that is pending (if any), then the read and the norm of sublayer `which`; returns the normed input."""
+        if pending is not None and not isinstance(pending, StreamsWrite):
+            raise TypeError("a streams block follows blocks of its own kind only")
+        norm = self.norms[which][1]
+        kw = {}
+        if pending is not None:
+            kw = dict(branch=pending.branch, mix=pending.mix, out_weights=pending.out)
+        return ops.streams_step(hidden, T, self.n, dtype=self.normed.dtype, read=self.hc[which][0], gain=norm.weight,
+                                bias=norm.bias, eps=norm.eps, out=self.normed, **kw)
+
+    def forward(self, hidden, pending, batch, cache: CacheView):
+        T = batch.num_tokens
+        if isinstance(pending, Carried):
+            pending = None
+        x = self._boundary(hidden, pending, 0, T)
+        a = self.mixer.forward(x, batch, cache)
+        pending = StreamsWrite(hidden, self.n, a, self.hc[0][1], self.hc[0][2])
+        if self.ff is not None:
+            x = self._boundary(hidden, pending, 1, T)
+            f = self.ff.forward(x, batch)
+            pending = StreamsWrite(hidden, self.n, f, self.hc[1][1], self.hc[1][2])
+        return pending

@@ -64,10 +64,12 @@ class GatedMLP(FeedForward):
 class MLP(FeedForward):
     """down( act(up(x)) ), no gate. act: a name of ops.ACTS."""
 
-    def __init__(self, hidden: int, intermediate: int, act: str = "relu2", names: tuple = ("up", "down")):
+    def __init__(self, hidden: int, intermediate: int, act: str = "relu2", names: tuple = ("up", "down"),
+                 out_name: str = "ffn_out", act_name: str = "act"):
         if act not in ops.ACTS:
             raise ValueError(f"feed-forward: activation {act!r} has no kernel (known: {sorted(ops.ACTS)})")
         self.hidden, self.intermediate, self.act, self.names = hidden, intermediate, act, tuple(names)
+        self.out_name, self.act_name = out_name, act_name
         self.up = Linear(hidden, intermediate)
         self.down = Linear(intermediate, hidden)
 
@@ -82,8 +84,8 @@ class MLP(FeedForward):
 
     def bind(self, ctx):
         ws = ctx.workspace
-        self.act_buf = ws.buffer("act", self.intermediate)
-        self.out_buf = ws.buffer("ffn_out", self.hidden)
+        self.act_buf = ws.buffer(self.act_name, self.intermediate)
+        self.out_buf = ws.buffer(self.out_name, self.hidden)
 
     def forward(self, x, batch, into=None):
         T = batch.num_tokens

@@ -146,7 +146,20 @@ class DecoderModel:
                 op.bind(ctx)
         ws = ctx.workspace
         stream = torch.float32 if self.spec.stream_dtype == "float32" else None
-        self.hidden = ws.buffer("hidden", self.spec.hidden_size, dtype=stream)
+        self.streams = int(self.spec.streams or 1)
+        if self.streams > 1:
+            # several residual streams a token: the embedding is gathered into a row of its own and copied into
+            # every stream; the sum of the streams of the wanted rows is what the final norm reads
+            if self.spec.stream_dtype != "float32":
+                raise ValueError("several residual streams are kept in float32 (stream_dtype)")
+            self.embedded_once = ws.buffer("embedded_once", self.spec.hidden_size, dtype=stream)
+            self.hidden = ws.buffer("hidden_streams", self.streams * self.spec.hidden_size, dtype=stream)
+            self.summed = ws.buffer("streams_summed", self.spec.hidden_size, dtype=stream, rows=ctx.max_rows)
+            self.ones = torch.ones(self.streams, dtype=torch.float32, device=ctx.device)
+            if self.keeps_embedding or self.embed_post is not None:
+                raise ValueError("several residual streams with operations on the embeddings are not built")
+        else:
+            self.hidden = ws.buffer("hidden", self.spec.hidden_size, dtype=stream)
         self.embedded = ws.buffer("embedded", self.spec.hidden_size, dtype=stream) if self.keeps_embedding else None
         self.final_normed = ws.buffer("final_normed", self.spec.hidden_size, rows=ctx.max_rows)
         self.logits = torch.empty((ctx.max_rows, self.spec.vocab_size), dtype=torch.float32, device=ctx.device)
@@ -155,8 +168,11 @@ class DecoderModel:
         """Runs the batch's tokens through all run entries; returns float32 logits [num_rows, vocab]
         at batch.logits_rows (a view of a fixed buffer)."""
         T, R = batch.num_tokens, batch.num_rows
-        ops.embedding(batch.input_ids[:T], self.embed, self.hidden, getattr(batch, "feedback_src", None),
+        first = self.hidden if self.streams == 1 else self.embedded_once
+        ops.embedding(batch.input_ids[:T], self.embed, first, getattr(batch, "feedback_src", None),
                       getattr(batch, "last_tokens", None), scale=self.spec.embed_scale)
+        if self.streams > 1:
+            ops.streams_expand(first, self.hidden, T, self.streams)
         if self.embed_post is not None:
             self.embed_post[1].forward(self.hidden, T)
         if self.embedded is not None:
@@ -171,6 +187,9 @@ class DecoderModel:
             if self.before[i] is not None:
                 # the stream must be whole before something is added to it from outside the blocks
                 if isinstance(pending, Carried):
+                    pending = None
+                elif hasattr(pending, "settle"):
+                    pending.settle(T)
                     pending = None
                 elif pending is not None:
                     ops.add_rows(self.hidden, T, a=pending)
@@ -188,7 +207,18 @@ class DecoderModel:
                 pending = block.forward(self.hidden, pending, batch, caches[i])
         if R == 0:
             return self.logits[:0]
-        if pending is None or isinstance(pending, Carried):
+        if self.streams > 1:
+            # the last write into the streams happens on the wanted rows only, inside the pass that sums them
+            kw = {}
+            if hasattr(pending, "settle"):
+                kw = dict(branch=pending.branch, mix=pending.mix, out_weights=pending.out)
+            ops.streams_step(self.hidden, R, self.streams, dtype=self.final_normed.dtype, read=self.ones,
+                             u_out=self.summed, rows=batch.logits_rows, **kw)
+            self.final_norm.forward(self.summed, self.final_normed, R)
+        elif hasattr(pending, "settle"):
+            pending.settle(T)
+            self.final_norm.forward(self.hidden, self.final_normed, R, rows=batch.logits_rows)
+        elif pending is None or isinstance(pending, Carried):
             self.final_norm.forward(self.hidden, self.final_normed, R, rows=batch.logits_rows)
         else:
             # the last add happens on the wanted rows only, inside the norm kernel

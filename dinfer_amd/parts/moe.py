@@ -5,6 +5,10 @@
     y = sum_chosen p_e * down_e( silu(gate_e x) * up_e x )
         + sigmoid(wsg . x) * shared(x)          (a gated feed-forward every token runs, where the layer has one)
 
+(The softmax over the chosen logits is the softmax over all experts with the chosen scores divided by their sum.)
+With `gated=False` an expert, and the shared one, is down_e( act(up_e x) ) with act "silu" or "gelu" (error function);
+with `shared_gate=False` the shared expert's output is added as it is.
+
 Per step: one kernel routes (logits, choice, weights, the shared gate), one sorts the (token, choice) entries by
 expert and writes the work list of row tiles, two launches run the products of all experts (gate and up with the
 activation, then down, each row computed alone and written to its entry's place), and one sums a token's entries in
@@ -18,7 +22,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward
-from .mlp import GatedMLP
+from .mlp import MLP, GatedMLP
 from .registry import FEED_FORWARDS
 from .spec import TensorSpec
 
@@ -29,40 +33,52 @@ class RoutedExperts(FeedForward):
     [1, hidden] where `shared_intermediate` is given."""
 
     def __init__(self, hidden: int, experts: int, top: int, intermediate: int, shared_intermediate: int | None = None,
-                 act: str = "silu"):
-        if act != "silu":
-            raise ValueError(f"routed feed-forward: activation {act!r} has no kernel (known: ['silu'])")
+                 act: str = "silu", gated: bool = True, shared_gate: bool = True):
+        if gated and act != "silu":
+            raise ValueError(f"routed feed-forward: gated activation {act!r} has no kernel (known: ['silu'])")
+        if not gated and act not in ops.EXPERT_ACTS:
+            raise ValueError(f"routed feed-forward: activation {act!r} has no kernel (known: {sorted(ops.EXPERT_ACTS)})")
         if not (0 < top <= experts) or experts > ops.MOE_MAX_EXPERTS or top > ops.MOE_MAX_TOP:
             raise ValueError(f"routed feed-forward: {top} of {experts} experts has no kernel (up to {ops.MOE_MAX_TOP} of "
                              f"{ops.MOE_MAX_EXPERTS})")
         self.hidden, self.experts, self.top, self.intermediate = hidden, experts, top, intermediate
+        self.gated, self.act, self.shared_gate_on = bool(gated), act, bool(shared_gate)
         self.shared = None
-        if shared_intermediate:
+        if shared_intermediate and gated:
             self.shared = GatedMLP(hidden, shared_intermediate, act, names=("shared.gate", "shared.up", "shared.down"),
                                    out_name="shared_out")
+        elif shared_intermediate:
+            self.shared = MLP(hidden, shared_intermediate, act, names=("shared.up", "shared.down"), out_name="shared_out",
+                              act_name="shared_act")
 
     def tensors(self):
         t = {"router": TensorSpec((self.experts, self.hidden))}
         for e in range(self.experts):
-            t[f"e{e}.gate"] = TensorSpec((self.intermediate, self.hidden))
+            if self.gated:
+                t[f"e{e}.gate"] = TensorSpec((self.intermediate, self.hidden))
             t[f"e{e}.up"] = TensorSpec((self.intermediate, self.hidden))
             t[f"e{e}.down"] = TensorSpec((self.hidden, self.intermediate))
         if self.shared is not None:
             t.update(self.shared.tensors())
-            t["shared.sg"] = TensorSpec((1, self.hidden))
+            if self.shared_gate_on:
+                t["shared.sg"] = TensorSpec((1, self.hidden))
         return t
 
     def load(self, get):
         self.router = get("router").float().contiguous()       # routing runs in 32 bits
         E = range(self.experts)
-        # [experts, 2 I, hidden]: an expert's gate rows, then its up rows; [experts, hidden, I]
-        self.w_in = torch.stack([torch.cat([get(f"e{e}.gate", compute=True), get(f"e{e}.up", compute=True)], dim=0)
-                                 for e in E]).contiguous()
+        # [experts, 2 I, hidden]: an expert's gate rows, then its up rows (not gated: [experts, I, hidden]); [experts, hidden, I]
+        if self.gated:
+            self.w_in = torch.stack([torch.cat([get(f"e{e}.gate", compute=True), get(f"e{e}.up", compute=True)], dim=0)
+                                     for e in E]).contiguous()
+        else:
+            self.w_in = torch.stack([get(f"e{e}.up", compute=True) for e in E]).contiguous()
         self.w_out = torch.stack([get(f"e{e}.down", compute=True) for e in E]).contiguous()
         self.sg = None
         if self.shared is not None:
             self.shared.load(get)
-            self.sg = get("shared.sg").float().reshape(-1).contiguous()
+            if self.shared_gate_on:
+                self.sg = get("shared.sg").float().reshape(-1).contiguous()
 
     def bind(self, ctx):
         ws, dev = ctx.workspace, ctx.device
@@ -88,9 +104,10 @@ class RoutedExperts(FeedForward):
         ops.moe_route(x, self.router, self.sg, self.idx, self.share, self.shared_gate, T, top, self.logits)
         rows = ops.moe_tile_rows(self.dtype, n, self.experts, self.hidden, self.intermediate)   # follows the step's count alone
         ops.moe_scatter(self.idx, n, self.experts, self.offsets, self.perm, self.tiles, rows)
-        ops.experts_nt(x, self.w_in, self.act_buf, n, self.tiles, self.offsets, self.perm, gated=True, a_div=top,
-                       c_to_perm=False, tile_rows=rows)
+        ops.experts_nt(x, self.w_in, self.act_buf, n, self.tiles, self.offsets, self.perm, gated=self.gated, a_div=top,
+                       c_to_perm=False, tile_rows=rows, act=None if self.gated else self.act)
         ops.experts_nt(self.act_buf, self.w_out, self.y_buf, n, self.tiles, self.offsets, self.perm, gated=False, a_div=0,
                        c_to_perm=True, tile_rows=rows)
         shared = self.shared.forward(x, batch) if self.shared is not None else None
-        return ops.moe_combine(self.y_buf, self.share, top, shared, self.shared_gate, self.out_buf, T)
+        return ops.moe_combine(self.y_buf, self.share, top, shared, self.shared_gate if self.sg is not None else None,
+                               self.out_buf, T)

@@ -30,7 +30,7 @@ class TensorSpec:
     """One tensor a part expects from the weight file.
 
     init: how the random-weights mode draws it: "linear" N(0, 0.02), "gain"
-    1 + N(0, 0.1), "zeros", "ones". keep_f32: stays 32-bit even in a bfloat16
+    1 + N(0, 0.1), "zeros", "ones", "eye" (the unit matrix). keep_f32: stays 32-bit even in a bfloat16
     engine when the file stores it so.
     """
     shape: tuple
@@ -168,8 +168,9 @@ class StateSpec(CacheSpec):
 
 @dataclass(frozen=True)
 class DeltaStateSpec(CacheSpec):
-    """Cache need of a delta-rule mixer: per request one float32 matrix a head, kept transposed [heads, vdim, dim],
-    and the last taps - 1 inputs of every channel of its short convolution, in the engine's dtype."""
+    """Cache need of a mixer whose state is one float32 matrix a head and request, kept transposed [heads, vdim, dim]
+    (the delta rule, a retention, a state-space mixer), and, where it has a short convolution, the last taps - 1 inputs
+    of every channel of it, in the engine's dtype (channels 0 and taps 1: none)."""
     heads: int
     dim: int
     vdim: int
@@ -279,3 +280,6 @@ class ModelSpec:
     # "float32": the residual stream is kept in 32 bits whatever the engine's dtype (the blocks' norms read it and write
     # the engine's dtype); None: the engine's dtype
     stream_dtype: str | None = None
+    # residual streams a token: with n > 1 the blocks are handed [T, n * hidden] (float32), the streams side by side,
+    # every one starting as the embedding; the final norm reads their sum
+    streams: int = 1

@@ -3,7 +3,7 @@ from a configuration and a seed.
 
 Every tensor is drawn from its own generator seeded by (seed, tensor name), so
 its values do not depend on the other tensors or on their order:
-matrix and table weights N(0, 0.02), norm gains 1 + N(0, 0.1). Values are drawn
+matrix and table weights N(0, 0.02), norm gains 1 + N(0, 0.1); "zeros", "ones" and "eye" (the unit matrix) are fixed. Values are drawn
 in float32 and stored in the requested dtype (bfloat16 by default).
 """
 from __future__ import annotations
@@ -39,6 +39,8 @@ def draw(seed: int, name: str, spec: TensorSpec, dtype: torch.dtype) -> torch.Te
         t = torch.zeros(spec.shape, dtype=torch.float32)
     elif spec.init == "ones":
         t = torch.ones(spec.shape, dtype=torch.float32)
+    elif spec.init == "eye":
+        t = torch.eye(*spec.shape, dtype=torch.float32)
     else:
         raise ValueError(f"tensor {name!r}: unknown init {spec.init!r}")
     return t.to(dtype)
@@ -48,7 +50,7 @@ def draw_on_device(seed: int, name: str, spec: TensorSpec, dtype: torch.dtype, d
     """The same rule as draw() (one generator per tensor, seeded by (seed, name); the same distributions), drawn by
     the device's generator: for measurements at sizes where a file would only cost time. The device's generator is
     another algorithm than the host's, so the values are not those of a folder written with the same seed."""
-    if spec.integer or spec.init in ("zeros", "ones"):
+    if spec.integer or spec.init in ("zeros", "ones", "eye"):
         return draw(seed, name, spec, dtype).to(device)
     g = torch.Generator(device=device)
     g.manual_seed(tensor_seed(seed, name))
