@@ -261,10 +261,9 @@ def random_weights(cfg, seed, scale=1.0):
     S = cfg.get("streams") or 1
     for name, shape in tensor_shapes(cfg).items():
         last = name.rsplit(".", 1)[-1]
-        if name.endswith(".b") and ".norm" in name or name.endswith("norm1.b") or name.endswith("norm2.b"):
-            x = 0.1 * torch.randn(shape, generator=g)
-        elif name.endswith(".b"):
-            x = 0.3 * torch.randn(shape, generator=g)
+        if name.endswith(".b"):          # a norm's bias is small, a projection's or a convolution's is not
+            of = name[:-2].rsplit(".", 1)[-1]
+            x = (0.1 if of.startswith("norm") else 0.3) * torch.randn(shape, generator=g)
         elif "norm" in last:
             x = 1.0 + 0.1 * torch.randn(shape, generator=g)
         elif last == "mix" and ".hc" in name:
@@ -284,7 +283,7 @@ def random_weights(cfg, seed, scale=1.0):
         elif name == "embed":
             x = torch.randn(shape, generator=g)
         elif last == "router":
-            x = 2.0 * torch.randn(shape, generator=g) / math.sqrt(shape[-1])
+            x = 6.0 * torch.randn(shape, generator=g) / math.sqrt(shape[-1])      # decisive: few tokens between two experts
         else:
             x = scale * 1.5 * torch.randn(shape, generator=g) / math.sqrt(shape[-1])
         w[name] = x.to(torch.bfloat16).to(F)
