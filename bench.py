@@ -6,6 +6,7 @@
     python bench.py --workload closed --shape 0.6b --concurrency 8 --prompt 128 --max-tokens 128 [--num-requests N]
     python bench.py --workload kudurax [--kudurax-shape 2k|4k] [--layers 4] [--prompt 2048] [--only kudurax|qwen3]
     python bench.py --workload karopel [--karopel-shape 2k|4k] [--layers 4] [--prompt 2048] [--only karopel|qwen3]
+    python bench.py --workload fanulix [--fanulix-shape 2k|4k] [--layers 4] [--prompt 2048] [--only fanulix|karopel|qwen3]
 
 Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
 request with a 2,048-token prompt in a 4,096-token context; a "step" is one decode step
@@ -256,6 +257,48 @@ def karopel_config(shape: dict, layers: int, vocab: int) -> dict:
                 norm=dict(eps=1e-6), loop=None, layers=[par if i % 4 in (1, 2) else att for i in range(layers)])
 
 
+# Fanulix layer sizes that resemble a real model's: a softmax attention with grouped keys and values beside a retention
+# of as many heads, all heads 128 wide; a state-space mixer of twice the width inside (heads of 64, state 128, 8 groups,
+# 4 taps); 64 routed experts of which a token uses 6, and a shared one; 4 residual streams. Beside them Karopel layers
+# of the same width (the closest design: an attention beside a recurrent mixer on one product each side) and Qwen3 layers
+FANULIX_SHAPES = {
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, ret_heads=16, ssm_heads=64, ssm_vdim=64, state=128, groups=8, conv=4,
+               norm_groups=8, experts=64, top=6, expert_ff=1408, shared_ff=2816, streams=4, karopel="2k",
+               qwen=dict(num_attention_heads=16, num_key_value_heads=4, head_dim=128, intermediate_size=8192)),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, ret_heads=32, ssm_heads=128, ssm_vdim=64, state=128, groups=8, conv=4,
+               norm_groups=8, experts=64, top=8, expert_ff=1536, shared_ff=3072, streams=4, karopel="4k",
+               qwen=dict(num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288)),
+}
+
+
+def fanulix_config(shape: dict, layers: int, vocab: int) -> dict:
+    """Layers in fours: parallel, state space, parallel, parallel; every layer with routed experts."""
+    d, rh = shape["dim"], shape["ret_heads"]
+    moe = dict(kind="moe", router=dict(experts=shape["experts"], top=shape["top"]), expert=dict(ff=shape["expert_ff"]),
+               shared=dict(ff=shape["shared_ff"]))
+    par = dict(type="parallel", mlp=moe, mixer=dict(
+        left=dict(heads=shape["heads"], kv_heads=shape["kv_heads"], dim=d, vdim=d, scale=d ** -0.5, q_temp=dict(coef=0.1, every=1024)),
+        right=dict(heads=rh, dim=d, vdim=d, decay=[1.0 - 2.0 ** (-5 - 3 * i / rh) for i in range(rh)],
+                   rot=dict(base=1000000.0, dims=d)),
+        left_scale=0.5, right_scale=0.5))
+    ssm = dict(type="mamba2", mlp=moe, mixer=dict(heads=shape["ssm_heads"], vdim=shape["ssm_vdim"], state=shape["state"],
+                                                   groups=shape["groups"], conv=shape["conv"], norm_groups=shape["norm_groups"]))
+    return dict(architecture="Fanulix", vocab=vocab, width=shape["width"], logit_scale=1.0, streams=shape["streams"],
+                norm=dict(eps=1e-5), layers=[ssm if i % 4 == 1 else par for i in range(layers)])
+
+
+def fanulix(a, torch, Engine, SamplingParams) -> int:
+    """Prefill and decode throughput of Fanulix layers of a real model's sizes beside Karopel and Qwen3 layers of the same
+    width."""
+    from dinfer_amd.config.fanulix import FanulixConfig
+    from dinfer_amd.config.karopel import KaropelConfig
+    shape = FANULIX_SHAPES[a.fanulix_shape]
+    layers = a.layers or 4
+    beside = {"karopel": KaropelConfig.from_dict(karopel_config(KAROPEL_SHAPES[shape["karopel"]], layers, 32768))}
+    return beside_qwen3(a, torch, Engine, SamplingParams, "fanulix", "Fanulix", a.fanulix_shape, shape,
+                        FanulixConfig.from_dict(fanulix_config(shape, layers, 32768)), beside=beside)
+
+
 def karopel(a, torch, Engine, SamplingParams) -> int:
     """Prefill and decode throughput of Karopel layers of a real model's sizes beside Qwen3 layers of the same width."""
     from dinfer_amd.config.karopel import KaropelConfig
@@ -275,13 +318,15 @@ def kudurax(a, torch, Engine, SamplingParams) -> int:
                         KuduraxConfig.from_dict(kudurax_config(shape, layers, 32768)))
 
 
-def beside_qwen3(a, torch, Engine, SamplingParams, key: str, label: str, shape_name: str, shape: dict, config) -> int:
+def beside_qwen3(a, torch, Engine, SamplingParams, key: str, label: str, shape_name: str, shape: dict, config,
+                 beside: dict | None = None) -> int:
     from dinfer_amd.config.qwen3 import Qwen3Config
     layers, vocab, page = a.layers or 4, 32768, 16
     PROMPT, CONTEXT = a.prompt, a.context
     batches = [b for b in (1, 8, 64) if b * CONTEXT <= 64 * 4096]
     models = {
         key: config,
+        **(beside or {}),
         "qwen3": Qwen3Config.from_dict({**SIZES, "vocab_size": vocab, "hidden_size": shape["width"],
                                         "num_hidden_layers": layers, **shape["qwen"]}),
     }
@@ -360,9 +405,10 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=DEFAULT_CONTEXT, help="max_model_len the engine is built for")
     ap.add_argument("--kudurax-shape", default="2k", choices=sorted(KUDURAX_SHAPES), help="kudurax: layer sizes")
     ap.add_argument("--karopel-shape", default="2k", choices=sorted(KAROPEL_SHAPES), help="karopel: layer sizes")
-    ap.add_argument("--only", default="", choices=["", "kudurax", "karopel", "qwen3"],
-                    help="kudurax, karopel: measure one of the two models")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed", "kudurax", "karopel"],
+    ap.add_argument("--fanulix-shape", default="2k", choices=sorted(FANULIX_SHAPES), help="fanulix: layer sizes")
+    ap.add_argument("--only", default="", choices=["", "kudurax", "karopel", "fanulix", "qwen3"],
+                    help="kudurax, karopel, fanulix: measure one of the models")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed", "kudurax", "karopel", "fanulix"],
                     help="serving: 32 requests with prompts of 512 to 3,072 tokens fed in portions of 512 beside the "
                          "requests that decode, 256 outputs each (meant for the 14B shape); closed: --concurrency "
                          "requests live at any time, --prompt tokens in and --max-tokens out each, the load of the "
@@ -388,6 +434,8 @@ def main() -> int:
         return kudurax(a, torch, Engine, SamplingParams)
     if a.workload == "karopel":
         return karopel(a, torch, Engine, SamplingParams)
+    if a.workload == "fanulix":
+        return fanulix(a, torch, Engine, SamplingParams)
     if a.workload == "serving":
         return serving(a, torch, Engine, SamplingParams, Qwen3Config)
     if a.workload == "closed":
