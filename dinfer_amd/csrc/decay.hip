@@ -9,7 +9,7 @@
 //   state space     q = C_t, k = B_t (shared by the heads of a group), v = x_t; a_t = exp(-exp(A) dt_t), c_t = dt_t;
 //                   x, B and C come out of a short causal convolution with bias and silu
 //
-//   rot_widen          one workgroup a token: q and k heads rotated (pairs (i, i + rot/2) of the first rot entries) by the
+//   rot_widen          a thread an entry: q and k heads rotated (pairs (i, i + rot/2) of the first rot entries) by the
 //                      table row of the token's position, k times a scale, v widened; float out
 //   conv_silu          a thread a (token, channel): taps over the step's rows and the request's stored inputs, bias, silu;
 //                      the threads behind the channels make dt = softplus(. + bias) and exp(-exp(A) dt) of every head
@@ -44,7 +44,7 @@ __device__ __forceinline__ int request_of(const int32_t* __restrict__ cu, int nu
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
-// work row: q (H D) | k (H D) | v (H V), float
+// work row: q (H D) | k (H D) | v (H V), float; a thread an entry
 template <class S>
 __global__ void __launch_bounds__(256) rot_widen_kernel(const S* __restrict__ proj, int64_t ld, int64_t q_off,
                                                         int64_t k_off, int64_t v_off, const int32_t* __restrict__ pos,
@@ -54,23 +54,26 @@ __global__ void __launch_bounds__(256) rot_widen_kernel(const S* __restrict__ pr
   const S* row = proj + t * ld;
   float* wr = work + t * ldw;
   const int half = rot / 2;
-  const float* cs = (cos_sin && rot > 0) ? cos_sin + (int64_t)pos[t] * rot : nullptr;
   const int hd = H * D;
-  for (int c = threadIdx.x; c < 2 * hd; c += blockDim.x) {
-    const bool is_k = c >= hd;
-    const int e = is_k ? c - hd : c;
-    const int d = e % D;
-    const S* src = row + (is_k ? k_off : q_off);
-    float y = to_f32(src[e]);
-    if (cs && d < rot) {
-      const bool first = d < half;
-      const int i = first ? d : d - half;
-      const float other = to_f32(src[first ? e + half : e - half]);
-      y = first ? rotated_first(y, other, cs[i], cs[half + i]) : rotated_second(other, y, cs[i], cs[half + i]);
-    }
-    wr[c] = is_k ? y * k_scale : y;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= 2 * hd + H * V) return;
+  if (c >= 2 * hd) {
+    wr[c] = to_f32(row[v_off + c - 2 * hd]);
+    return;
   }
-  for (int c = threadIdx.x; c < H * V; c += blockDim.x) wr[2 * hd + c] = to_f32(row[v_off + c]);
+  const bool is_k = c >= hd;
+  const int e = is_k ? c - hd : c;
+  const int d = e % D;
+  const S* src = row + (is_k ? k_off : q_off);
+  float y = to_f32(src[e]);
+  if (cos_sin && d < rot) {
+    const float* cs = cos_sin + (int64_t)pos[t] * rot;
+    const bool first = d < half;
+    const int i = first ? d : d - half;
+    const float other = to_f32(src[first ? e + half : e - half]);
+    y = first ? rotated_first(y, other, cs[i], cs[half + i]) : rotated_second(other, y, cs[i], cs[half + i]);
+  }
+  wr[c] = is_k ? y * k_scale : y;
 }
 
 // work row: the C channels after convolution, bias and silu | dt (H) | decay (H), float
@@ -193,17 +196,31 @@ __global__ void __launch_bounds__(256) decay_recurrence_kernel(Operands p, float
     __syncthreads();
     if (ct + CH < n) fetch(ct + CH);  // in flight while this chunk is worked through
     const int m = n - ct < CH ? n - ct : CH;
-    for (int tok = 0; tok < m; ++tok) {
-      const float a = as[tok], vt = vs[tok][cj];
-      float o0 = 0.f, o1 = 0.f;   // two chains: a fixed order all the same
+    // four tokens a round: only the state's update runs from token to token, the four row sums meet the lanes
+    // together (places behind the step's last token hold k = 0, v = 0 and a decay of one, and change nothing)
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        S[i] = __builtin_fmaf(ks[tok][rg * RPT + i], vt, a * S[i]);
-        if (i & 1) o1 = __builtin_fmaf(S[i], qs[tok][rg * RPT + i], o1);
-        else o0 = __builtin_fmaf(S[i], qs[tok][rg * RPT + i], o0);
+    for (int t4 = 0; t4 < CH; t4 += 4) {
+      if (t4 >= m) break;
+      float part[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int tok = t4 + u;
+        const float a = as[tok], vt = vs[tok][cj];
+        float o0 = 0.f, o1 = 0.f;   // two chains: a fixed order all the same
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+          S[i] = __builtin_fmaf(ks[tok][rg * RPT + i], vt, a * S[i]);
+          if (i & 1) o1 = __builtin_fmaf(S[i], qs[tok][rg * RPT + i], o1);
+          else o0 = __builtin_fmaf(S[i], qs[tok][rg * RPT + i], o0);
+        }
+        part[u] = o0 + o1;
       }
-      const float o = half_wave_sum(o0 + o1);
-      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * V + j] = o;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) part[u] = half_wave_sum(part[u]);
+      if (rg < 4 && col_ok && t4 + rg < m) {
+        const float o = rg == 0 ? part[0] : rg == 1 ? part[1] : rg == 2 ? part[2] : part[3];
+        out[(int64_t)(t0 + ct + t4 + rg) * ld_out + h * V + j] = o;
+      }
     }
   }
   if (col_ok) {
@@ -256,8 +273,9 @@ extern "C" int dinfer_rot_widen(int dtype, const void* proj, int64_t ld, int64_t
   if (H <= 0 || D <= 0 || V <= 0 || rot < 0 || rot > D || rot % 2 || tokens > 0x7fffffff ||
       ldw < 2 * (int64_t)H * D + (int64_t)H * V)
     return ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)tokens, (unsigned)((2 * H * D + H * V + 255) / 256));
   DINFER_DISPATCH_DTYPE(dtype, {
-    rot_widen_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)proj, ld, q_off, k_off, v_off, positions, cos_sin,
+    rot_widen_kernel<S><<<grid, 256, 0, stream>>>((const S*)proj, ld, q_off, k_off, v_off, positions, cos_sin,
                                                               rot, k_scale, work, ldw, H, D, V);
   });
   return launch_status();

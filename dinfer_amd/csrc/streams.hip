@@ -7,7 +7,7 @@
 //   x_t <- sum_s m[s, t] x_s + o[t] y      all streams at once from the old ones, y the sublayer's output
 //
 //   streams_expand   every stream of a token starts as the same row (the embedding)
-//   streams_step     one workgroup a token does what lies between two sublayers in one pass over the row: the write of
+//   streams_step     one workgroup a token (the number of streams a template parameter, 16-byte moves) does what lies between two sublayers in one pass over the row: the write of
 //                    the sublayer that has just run (optional), the read for the one that runs next (optional), and
 //                    that one's layer norm with gain and bias (optional; without it u is written as float). With a list
 //                    of source rows (the rows whose logits are wanted) nothing is stored into the streams.
@@ -42,55 +42,79 @@ struct Step {
   float* u_out; int64_t ld_u;
 };
 
-template <class S>
+// N streams (a template parameter: every array below stays in registers), VEC consecutive columns a thread and pass.
+template <class S, int N, int VEC>
 __global__ void __launch_bounds__(256) streams_step_kernel(Step p) {
   extern __shared__ float us[];              // u of this row
   __shared__ float red[16];
-  __shared__ float mix_s[MAX_STREAMS * MAX_STREAMS], out_s[MAX_STREAMS], read_s[MAX_STREAMS];
-  const int n = p.n, W = p.width;
-  if (threadIdx.x < n * n && p.branch) mix_s[threadIdx.x] = p.mix[threadIdx.x];
-  if (threadIdx.x < n) {
-    out_s[threadIdx.x] = p.branch ? p.outw[threadIdx.x] : 0.f;
-    read_s[threadIdx.x] = p.read ? p.read[threadIdx.x] : 0.f;
+  const int W = p.width;
+  float mix[N][N], outw[N], readw[N];
+#pragma unroll
+  for (int s = 0; s < N; ++s) {
+    outw[s] = p.branch ? p.outw[s] : 0.f;
+    readw[s] = p.read ? p.read[s] : 0.f;
+#pragma unroll
+    for (int to = 0; to < N; ++to) mix[s][to] = p.branch ? p.mix[s * N + to] : 0.f;
   }
-  __syncthreads();
   const int64_t r = blockIdx.x;
   const int64_t t = p.rows ? p.rows[r] : r;
   float* xr = p.x + t * p.ldx;
   const S* y = p.branch ? (const S*)p.branch + t * p.ld_branch : nullptr;
   float sum = 0.f;
-  for (int c = threadIdx.x; c < W; c += 256) {
-    float xs[MAX_STREAMS];
+  for (int c = threadIdx.x * VEC; c < W; c += 256 * VEC) {
+    float xs[N][VEC];
 #pragma unroll
-    for (int s = 0; s < MAX_STREAMS; ++s) xs[s] = s < n ? xr[(int64_t)s * W + c] : 0.f;
-    if (y) {
-      const float yv = to_f32(y[c]);
-      float nx[MAX_STREAMS];
+    for (int s = 0; s < N; ++s) {
+      if (VEC == 4) {
+        const f32x4 v = *(const f32x4*)(xr + (int64_t)s * W + c);
 #pragma unroll
-      for (int to = 0; to < MAX_STREAMS; ++to) {
-        float acc = 0.f;
-        if (to < n) {
-          for (int s = 0; s < n; ++s) acc = __builtin_fmaf(mix_s[s * n + to], xs[s], acc);
-          acc = __builtin_fmaf(out_s[to], yv, acc);
-        }
-        nx[to] = acc;
+        for (int e = 0; e < VEC; ++e) xs[s][e] = v[e];
+      } else {
+        xs[s][0] = xr[(int64_t)s * W + c];
       }
+    }
+    if (y) {
+      float yv[VEC];
 #pragma unroll
-      for (int s = 0; s < MAX_STREAMS; ++s) {
-        xs[s] = nx[s];
-        if (s < n && !p.rows) xr[(int64_t)s * W + c] = nx[s];
+      for (int e = 0; e < VEC; ++e) yv[e] = to_f32(y[c + e]);
+      float nx[N][VEC];
+#pragma unroll
+      for (int to = 0; to < N; ++to)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          float acc = 0.f;
+#pragma unroll
+          for (int s = 0; s < N; ++s) acc = __builtin_fmaf(mix[s][to], xs[s][e], acc);
+          nx[to][e] = __builtin_fmaf(outw[to], yv[e], acc);
+        }
+#pragma unroll
+      for (int s = 0; s < N; ++s) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) xs[s][e] = nx[s][e];
+        if (!p.rows) {
+          if (VEC == 4) {
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] = nx[s][e];
+            *(f32x4*)(xr + (int64_t)s * W + c) = v;
+          } else {
+            xr[(int64_t)s * W + c] = nx[s][0];
+          }
+        }
       }
     }
     if (p.read) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < MAX_STREAMS; ++s)
-        if (s < n) u = __builtin_fmaf(read_s[s], xs[s], u);
-      if (p.gain) {
-        us[c] = u;
-        sum += u;
-      } else {
-        p.u_out[r * p.ld_u + c] = u;
+      for (int e = 0; e < VEC; ++e) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < N; ++s) u = __builtin_fmaf(readw[s], xs[s][e], u);
+        if (p.gain) {
+          us[c + e] = u;
+          sum += u;
+        } else {
+          p.u_out[r * p.ld_u + c + e] = u;
+        }
       }
     }
   }
@@ -105,6 +129,21 @@ __global__ void __launch_bounds__(256) streams_step_kernel(Step p) {
   S* o = (S*)p.out + r * p.ld_out;
   for (int c = threadIdx.x; c < W; c += 256)
     o[c] = from_f32<S>((us[c] - mean) * inv * p.gain[c] + (p.bias ? p.bias[c] : 0.f));
+}
+
+template <class S, int VEC>
+void launch_step(const Step& p, int64_t n_rows, size_t lds, hipStream_t stream) {
+  const unsigned g = (unsigned)n_rows;
+  switch (p.n) {
+    case 1: streams_step_kernel<S, 1, VEC><<<g, 256, lds, stream>>>(p); break;
+    case 2: streams_step_kernel<S, 2, VEC><<<g, 256, lds, stream>>>(p); break;
+    case 3: streams_step_kernel<S, 3, VEC><<<g, 256, lds, stream>>>(p); break;
+    case 4: streams_step_kernel<S, 4, VEC><<<g, 256, lds, stream>>>(p); break;
+    case 5: streams_step_kernel<S, 5, VEC><<<g, 256, lds, stream>>>(p); break;
+    case 6: streams_step_kernel<S, 6, VEC><<<g, 256, lds, stream>>>(p); break;
+    case 7: streams_step_kernel<S, 7, VEC><<<g, 256, lds, stream>>>(p); break;
+    default: streams_step_kernel<S, 8, VEC><<<g, 256, lds, stream>>>(p); break;
+  }
 }
 
 }  // namespace
@@ -134,6 +173,11 @@ extern "C" int dinfer_streams_step(int dtype, float* x, int64_t ldx, int n, int 
   if (!branch && !read) return OK;
   Step p{x, ldx, n, width, rows, branch, ld_branch, mix, outw, read, gain, bias, eps, out, ld_out, u_out, ld_u};
   const size_t lds = (read && gain) ? (size_t)width * sizeof(float) : 0;
-  DINFER_DISPATCH_DTYPE(dtype, { streams_step_kernel<S><<<(unsigned)n_rows, 256, lds, stream>>>(p); });
+  // 16-byte moves where every stream of every row starts on a 16-byte boundary
+  const bool vec = width % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)x % 16) == 0;
+  DINFER_DISPATCH_DTYPE(dtype, {
+    if (vec) launch_step<S, 4>(p, n_rows, lds, stream);
+    else launch_step<S, 1>(p, n_rows, lds, stream);
+  });
   return launch_status();
 }
