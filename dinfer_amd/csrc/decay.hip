@@ -144,18 +144,33 @@ __global__ void __launch_bounds__(256) decay_recurrence_kernel(Operands p, float
   __shared__ __attribute__((aligned(16))) float qs[CH][DP];
   __shared__ float vs[CH][COLS];
   __shared__ float as[CH];
-  const int b = blockIdx.x, h = blockIdx.y;
+  // the request is the slowest index of the grid: the workgroups of one long request among many short ones then
+  // spread over all XCDs (consecutive workgroups go to consecutive XCDs) instead of meeting on one
+  const int b = blockIdx.z, h = blockIdx.y, cb = blockIdx.x;
   const int tid = threadIdx.x;
   const int rg = tid & 31, cj = tid >> 5;
-  const int j = blockIdx.z * COLS + cj;
+  const int j = cb * COLS + cj;
   const int t0 = cu[b], n = cu[b + 1] - t0;
   const int start = seq_lens[b] - n;
   const int g = h / (H / G);
   const bool col_ok = j < V;
   float* sp = state + ((((int64_t)slots[b] * H + h) * V + (col_ok ? j : 0)) * D) + rg * RPT;
   float S[RPT];
+  // a strip of a multiple of 4 rows in a matrix of a multiple of 4 rows moves 16 bytes at a time
+  const bool quads = RPT % 4 == 0 && D % 4 == 0;
+  if (quads) {
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) S[i] = (start > 0 && col_ok && rg * RPT + i < D) ? sp[i] : 0.f;
+    for (int i = 0; i < RPT; i += 4) {
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (start > 0 && col_ok && rg * RPT + i < D) v = *(const f32x4*)(sp + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (i + e < RPT) S[i + e] = v[e];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) S[i] = (start > 0 && col_ok && rg * RPT + i < D) ? sp[i] : 0.f;
+  }
 
   // what a thread carries of the next chunk: entries of k and of q, one of v (times its step size), one decay
   constexpr int PK = (CH * DP) / 256;
@@ -172,7 +187,7 @@ __global__ void __launch_bounds__(256) decay_recurrence_kernel(Operands p, float
     }
     if (tid < CH * COLS) {
       const int tok = tid / COLS, c = tid % COLS;
-      const int col = blockIdx.z * COLS + c;
+      const int col = cb * COLS + c;
       const int64_t t = t0 + ct + tok;
       pv = 0.f;
       if (ct + tok < n && col < V) {
@@ -197,10 +212,9 @@ __global__ void __launch_bounds__(256) decay_recurrence_kernel(Operands p, float
     if (ct + CH < n) fetch(ct + CH);  // in flight while this chunk is worked through
     const int m = n - ct < CH ? n - ct : CH;
     // four tokens a round: only the state's update runs from token to token, the four row sums meet the lanes
-    // together (places behind the step's last token hold k = 0, v = 0 and a decay of one, and change nothing)
-#pragma unroll
-    for (int t4 = 0; t4 < CH; t4 += 4) {
-      if (t4 >= m) break;
+    // together; what is left of the step's rows (all of a single decoded row) goes token by token
+    int t4 = 0;
+    for (; t4 + 4 <= m; t4 += 4) {
       float part[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
@@ -217,13 +231,33 @@ __global__ void __launch_bounds__(256) decay_recurrence_kernel(Operands p, float
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) part[u] = half_wave_sum(part[u]);
-      if (rg < 4 && col_ok && t4 + rg < m) {
+      if (rg < 4 && col_ok) {
         const float o = rg == 0 ? part[0] : rg == 1 ? part[1] : rg == 2 ? part[2] : part[3];
         out[(int64_t)(t0 + ct + t4 + rg) * ld_out + h * V + j] = o;
       }
     }
+    for (int tok = t4; tok < m; ++tok) {
+      const float a = as[tok], vt = vs[tok][cj];
+      float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        S[i] = __builtin_fmaf(ks[tok][rg * RPT + i], vt, a * S[i]);
+        if (i & 1) o1 = __builtin_fmaf(S[i], qs[tok][rg * RPT + i], o1);
+        else o0 = __builtin_fmaf(S[i], qs[tok][rg * RPT + i], o0);
+      }
+      const float o = half_wave_sum(o0 + o1);
+      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * V + j] = o;
+    }
   }
-  if (col_ok) {
+  if (col_ok && quads) {
+#pragma unroll
+    for (int i = 0; i < RPT; i += 4) {
+      f32x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = S[i + e < RPT ? i + e : 0];
+      if (rg * RPT + i < D) *(f32x4*)(sp + i) = v;
+    }
+  } else if (col_ok) {
 #pragma unroll
     for (int i = 0; i < RPT; ++i)
       if (rg * RPT + i < D) sp[i] = S[i];
@@ -309,10 +343,10 @@ extern "C" int dinfer_decay_recurrence(const float* q, int64_t ldq, const float*
                                        const int32_t* cu_seqlens, const int32_t* seq_lens, float* out, int64_t ld_out,
                                        int num_reqs, int G, int H, int D, int V, hipStream_t stream) {
   if (num_reqs <= 0) return OK;
-  if (G <= 0 || H <= 0 || H % G || D <= 0 || V <= 0 || num_reqs > 0x7fffffff || H > 65535 || !decay) return ERR_BAD_SHAPE;
+  if (G <= 0 || H <= 0 || H % G || D <= 0 || V <= 0 || num_reqs > 65535 || H > 65535 || !decay) return ERR_BAD_SHAPE;
   if (D > 256) return ERR_UNSUPPORTED;
   Operands p{q, ldq, k, ldk, v, ldv, decay, ld_decay, gain, ld_gain};
-  const dim3 grid((unsigned)num_reqs, (unsigned)H, (unsigned)((V + COLS - 1) / COLS));
+  const dim3 grid((unsigned)((V + COLS - 1) / COLS), (unsigned)H, (unsigned)num_reqs);
 #define DECAY_REC(R_) \
   decay_recurrence_kernel<R_><<<grid, 256, 0, stream>>>(p, state, state_slots, cu_seqlens, seq_lens, out, ld_out, G, H, D, V)
   if (D <= 32) DECAY_REC(1);

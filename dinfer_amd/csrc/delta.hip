@@ -241,10 +241,12 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
   __shared__ __attribute__((aligned(16))) float qs[CH][DP];
   __shared__ float vs[CH][COLS];
   __shared__ float bs[CH], gs[CH];
-  const int b = blockIdx.x, h = blockIdx.y;
+  // the request is the slowest index of the grid: the workgroups of one long request among many short ones then
+  // spread over all XCDs (consecutive workgroups go to consecutive XCDs) instead of meeting on one
+  const int b = blockIdx.z, h = blockIdx.y, cb = blockIdx.x;
   const int tid = threadIdx.x;
   const int rg = tid & 31, cj = tid >> 5;
-  const int j = blockIdx.z * COLS + cj;
+  const int j = cb * COLS + cj;
   const int t0 = cu[b], n = cu[b + 1] - t0;
   const int start = seq_lens[b] - n;
   const int g = h / (H / G);
@@ -271,7 +273,7 @@ __global__ void __launch_bounds__(256) delta_recurrence_kernel(
     }
     if (tid < CH * COLS) {
       const int tok = tid / COLS, c = tid % COLS;
-      const int col = blockIdx.z * COLS + c;
+      const int col = cb * COLS + c;
       pv = (ct + tok < n && col < V) ? wk[(int64_t)(ct + tok) * ldw + gd + h * V + col] : 0.f;
     }
     if (tid < 2 * CH) {
@@ -430,9 +432,9 @@ extern "C" int dinfer_delta_recurrence(const float* work, int64_t ldw, float* st
                                        const int32_t* cu_seqlens, const int32_t* seq_lens, float* out, int64_t ld_out,
                                        int num_reqs, int G, int H, int D, int V, hipStream_t stream) {
   if (num_reqs <= 0) return OK;
-  if (G <= 0 || H <= 0 || H % G || D <= 0 || V <= 0 || num_reqs > 0x7fffffff || H > 65535) return ERR_BAD_SHAPE;
+  if (G <= 0 || H <= 0 || H % G || D <= 0 || V <= 0 || num_reqs > 65535 || H > 65535) return ERR_BAD_SHAPE;
   if (D > 256) return ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)num_reqs, (unsigned)H, (unsigned)((V + COLS - 1) / COLS));
+  const dim3 grid((unsigned)((V + COLS - 1) / COLS), (unsigned)H, (unsigned)num_reqs);
 #define DELTA_REC(R_)                                                                                               \
   delta_recurrence_kernel<R_><<<grid, 256, 0, stream>>>(work, ldw, state, state_slots, cu_seqlens, seq_lens, out, \
                                                         ld_out, G, H, D, V)
