@@ -283,11 +283,33 @@ __global__ void __launch_bounds__(256) gated_group_norm_kernel(const float* __re
     return gate_first ? u * silu_f(to_f32(z[t * ld_z + z_off + c])) : u;
   };
   float ss = 0.f;
-  for (int c = c0 + threadIdx.x; c < c0 + group; c += 256) {
-    const float u = value(c);
-    ss = __builtin_fmaf(u, u, ss);
+  constexpr int KEEP = 4;                    // a group of up to 1,024 columns stays in registers between the two passes
+  float kept[KEEP];
+  const bool keeps = group <= 256 * KEEP;
+#pragma unroll
+  for (int e = 0; e < KEEP; ++e) {
+    const int c = c0 + threadIdx.x + 256 * e;
+    kept[e] = (keeps && c < c0 + group) ? value(c) : 0.f;
+    ss = __builtin_fmaf(kept[e], kept[e], ss);
   }
+  if (!keeps)
+    for (int c = c0 + threadIdx.x; c < c0 + group; c += 256) {
+      const float u = value(c);
+      ss = __builtin_fmaf(u, u, ss);
+    }
   const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)group + eps);
+  if (keeps) {
+#pragma unroll
+    for (int e = 0; e < KEEP; ++e) {
+      const int c = c0 + threadIdx.x + 256 * e;
+      if (c < c0 + group) {
+        float r = kept[e] * inv * (w ? w[c] : 1.f) * out_scale;
+        if (!gate_first) r *= silu_f(to_f32(z[t * ld_z + z_off + c]));
+        out[t * ld_out + col_off + c] = from_f32<S>(r);
+      }
+    }
+    return;
+  }
   for (int c = c0 + threadIdx.x; c < c0 + group; c += 256) {
     float r = value(c) * inv * (w ? w[c] : 1.f) * out_scale;
     if (!gate_first) r *= silu_f(to_f32(z[t * ld_z + z_off + c]));

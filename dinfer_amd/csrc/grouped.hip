@@ -359,6 +359,40 @@ __global__ void __launch_bounds__(256) moe_logits_kernel(const S* __restrict__ x
   }
 }
 
+// The same for bfloat16 rows of a width that is a multiple of 8: a lane takes 8 consecutive entries at a time (16-byte
+// loads of x, two of the router's row), so a token costs an eighth of the load instructions.
+template <int RT>
+__global__ void __launch_bounds__(256) moe_logits_bf16x8_kernel(const bf16* __restrict__ x, int64_t ld_x, int tokens,
+                                                                const float* __restrict__ wr, const float* __restrict__ wsg,
+                                                                int E, int width, float* __restrict__ z, int ldz) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int e = blockIdx.y * 4 + wave;
+  if (e >= E + (wsg ? 1 : 0)) return;
+  const float* w = e < E ? wr + (int64_t)e * width : wsg;
+  const int t0 = blockIdx.x * RT;
+  const int nt = tokens - t0 < RT ? tokens - t0 : RT;
+  float acc[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc[r] = 0.f;
+  for (int i = lane * 8; i < width; i += 512) {
+    const f32x4 w0 = *(const f32x4*)(w + i), w1 = *(const f32x4*)(w + i + 4);
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+      if (r < nt) {
+        const bf16x8 v = *(const bf16x8*)(x + (int64_t)(t0 + r) * ld_x + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[r] = fmaf((float)v[j], w0[j], acc[r]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[r] = fmaf((float)v[4 + j], w1[j], acc[r]);
+      }
+  }
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const float v = wave_sum(acc[r]);
+    if (lane == 0 && r < nt) z[(int64_t)(t0 + r) * ldz + e] = v;
+  }
+}
+
 // A wave per token: the `top` largest of its logits, one after the other (among equals the lowest index), the softmax
 // over the chosen, and the sigmoid of the shared expert's gate logit (z[t, E]) where there is one.
 __global__ void __launch_bounds__(256) moe_topk_kernel(const float* __restrict__ z, int ldz, int tokens, int E, int top,
@@ -564,6 +598,16 @@ extern "C" int dinfer_moe_route(int dtype, const void* x, int64_t ld_x, int64_t 
   const int rows = experts + (shared_gate_w ? 1 : 0), ldz = experts + 1;
   const int rt = tokens <= 128 ? 1 : 8;
   const dim3 grid((unsigned)((tokens + rt - 1) / rt), (unsigned)((rows + 3) / 4));
+  const bool x8 = dtype == DT_BF16 && width % 8 == 0 && ld_x % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
+                  ((uintptr_t)router % 16) == 0 && ((uintptr_t)shared_gate_w % 16) == 0;
+  if (x8) {
+    if (rt == 1)
+      moe_logits_bf16x8_kernel<1><<<grid, 256, 0, stream>>>((const bf16*)x, ld_x, (int)tokens, router, shared_gate_w,
+                                                            experts, width, z, ldz);
+    else
+      moe_logits_bf16x8_kernel<8><<<grid, 256, 0, stream>>>((const bf16*)x, ld_x, (int)tokens, router, shared_gate_w,
+                                                            experts, width, z, ldz);
+  } else
   DINFER_DISPATCH_DTYPE(dtype, {
     if (rt == 1)
       moe_logits_kernel<S, 1><<<grid, 256, 0, stream>>>((const S*)x, ld_x, (int)tokens, router, shared_gate_w, experts,
