@@ -109,6 +109,71 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(
   wr[c] = silu_f(acc);
 }
 
+// The same for bfloat16 rows and K taps known when compiled: a thread takes 8 consecutive channels of a token, so a
+// row's inputs come as one 16-byte load a tap (the K rows are asked for before the first is used), the 8 K taps of
+// its channels are consecutive floats, and the result leaves as two 16-byte stores. The stored inputs of a request
+// ([channel][K - 1]) are read one value at a time: only the first K - 1 rows of a request's portion need them.
+template <int K>
+__global__ void __launch_bounds__(256) conv_silu_vec_kernel(
+    const bf16* __restrict__ proj, int64_t ld, int64_t x_off, int64_t dt_off, const float* __restrict__ taps,
+    const float* __restrict__ bias, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    const bf16* __restrict__ conv_state, const int32_t* __restrict__ slots, const int32_t* __restrict__ cu,
+    const int32_t* __restrict__ seq_lens, float* __restrict__ work, int64_t ldw, int num_reqs, int C, int H) {
+  const int t = blockIdx.x;
+  const int u = blockIdx.y * 256 + threadIdx.x;
+  const int pieces = C / 8;
+  if (u >= pieces + H) return;
+  const bf16* row = proj + (int64_t)t * ld;
+  float* wr = work + (int64_t)t * ldw;
+  if (u >= pieces) {
+    const int h = u - pieces;
+    const float dt = softplus_f((float)row[dt_off + h] + dt_bias[h]);
+    wr[C + h] = dt;
+    wr[C + H + h] = expf(-expf(a_log[h]) * dt);
+    return;
+  }
+  const int c = 8 * u;
+  const int b = request_of(cu, num_reqs, t);
+  const int i = t - cu[b];
+  const int start = seq_lens[b] - (cu[b + 1] - cu[b]);
+  const bf16* old = (K > 1 && start > 0) ? conv_state + (int64_t)slots[b] * C * (K - 1) : nullptr;
+  bf16x8 in[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    if (i - j >= 0) {
+      in[j] = *(const bf16x8*)(row + x_off + c - (int64_t)j * ld);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        in[j][e] = old ? old[(int64_t)(c + e) * (K - 1) + (K - 1 + i - j)] : (bf16)0.f;
+    }
+  }
+  float tap[8 * K];
+#pragma unroll
+  for (int e = 0; e < 2 * K; ++e) {
+    const f32x4 w = *(const f32x4*)(taps + (int64_t)c * K + 4 * e);
+    tap[4 * e] = w[0]; tap[4 * e + 1] = w[1]; tap[4 * e + 2] = w[2]; tap[4 * e + 3] = w[3];
+  }
+  float acc[8];
+  if (bias) {
+    const f32x4 b0 = *(const f32x4*)(bias + c), b1 = *(const f32x4*)(bias + c + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { acc[e] = b0[e]; acc[4 + e] = b1[e]; }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  }
+#pragma unroll
+  for (int j = K - 1; j >= 0; --j)                           // the oldest input first, as the kernel above
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(tap[e * K + (K - 1 - j)], (float)in[j][e], acc[e]);
+  f32x4 o0, o1;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { o0[e] = silu_f(acc[e]); o1[e] = silu_f(acc[4 + e]); }
+  *(f32x4*)(wr + c) = o0;
+  *(f32x4*)(wr + c + 4) = o1;
+}
+
 // A lane's value plus that of the lane a DPP pattern pairs it with (full-rate vector instructions, no LDS).
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
@@ -348,6 +413,21 @@ extern "C" int dinfer_conv_silu(int dtype, const void* proj, int64_t ld, int64_t
   if (tokens <= 0 || num_reqs <= 0) return OK;
   if (C <= 0 || H <= 0 || K <= 0 || tokens > 0x7fffffff || ldw < (int64_t)C + 2 * H) return ERR_BAD_SHAPE;
   if (K > MAX_TAPS) return ERR_UNSUPPORTED;
+  const bool vec = dtype == DT_BF16 && K >= 2 && K <= 4 && C % 8 == 0 && ld % 8 == 0 && x_off % 8 == 0 && ldw % 4 == 0 &&
+                   ((uintptr_t)proj % 16) == 0 && ((uintptr_t)work % 16) == 0 && ((uintptr_t)taps % 16) == 0 &&
+                   ((uintptr_t)bias % 16) == 0;
+  if (vec) {
+    const dim3 vgrid((unsigned)tokens, (unsigned)((C / 8 + H + 255) / 256));
+#define DINFER_CONV_VEC(K_)                                                                                          \
+  conv_silu_vec_kernel<K_><<<vgrid, 256, 0, stream>>>((const bf16*)proj, ld, x_off, dt_off, taps, bias, a_log, dt_bias, \
+                                                      (const bf16*)conv_state, state_slots, cu_seqlens, seq_lens, work, \
+                                                      ldw, num_reqs, C, H)
+    if (K == 2) DINFER_CONV_VEC(2);
+    else if (K == 3) DINFER_CONV_VEC(3);
+    else DINFER_CONV_VEC(4);
+#undef DINFER_CONV_VEC
+    return launch_status();
+  }
   const dim3 grid((unsigned)tokens, (unsigned)((C + H + 255) / 256));
   DINFER_DISPATCH_DTYPE(dtype, {
     conv_silu_kernel<S><<<grid, 256, 0, stream>>>((const S*)proj, ld, x_off, dt_off, taps, bias, a_log, dt_bias,

@@ -236,7 +236,8 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_neox_kernel(
 // (group: which run of 8 * WAVES tokens the workgroup takes.)
 __device__ __forceinline__ void v_write_transposed(const bf16* __restrict__ qkv, int64_t ld, int64_t v_off,
                                                    bf16* __restrict__ v_cache, const int64_t* __restrict__ slots, int T,
-                                                   int Hkv, int D, int page, int group, int hk) {
+                                                   int Hkv, int D, int page, int group, int hk,
+                                                   const float* __restrict__ vb = nullptr) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t0 = (group * WAVES + wave) * 8;
   if (t0 >= T) return;
@@ -250,6 +251,15 @@ __device__ __forceinline__ void v_write_transposed(const bf16* __restrict__ qkv,
 #pragma unroll
     for (int j = 0; j < 8; ++j)
       if (j < n) v[j] = *(const bf16x2*)(src + (int64_t)j * ld + 2 * d2);
+    if (vb) {  // the head's bias (float), added as the kernels that take one value at a time add it
+      const float b0 = vb[2 * d2], b1 = vb[2 * d2 + 1];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (j < n) {
+          v[j][0] = (bf16)((float)v[j][0] + b0);
+          v[j][1] = (bf16)((float)v[j][1] + b1);
+        }
+    }
     if (aligned) {
       const int64_t blk = s0 / page;
       const int off = (int)(s0 % page);
@@ -288,11 +298,14 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
     bf16* __restrict__ qkv, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, const void* __restrict__ wq,
     const void* __restrict__ wk, int wf32, float eps, float w_offset, const int32_t* __restrict__ pos,
     const float* __restrict__ cos_sin, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
-    const int64_t* __restrict__ slots, int H, int Hkv, int page, int tokens, int gather_v) {
+    const int64_t* __restrict__ slots, int H, int Hkv, int page, int tokens, int gather_v,
+    const float* __restrict__ bias, float temp_coef, int temp_every) {
   constexpr int D = LPH * 8, HALF = D / 2, HPW = 64 / LPH;  // heads per wave
   if ((int)blockIdx.x >= tokens) {
     const int j = (int)blockIdx.x - tokens;
-    if (blockIdx.y == 0) v_write_transposed(qkv, ld, v_off, v_cache, slots, tokens, Hkv, D, page, j / Hkv, j % Hkv);
+    if (blockIdx.y == 0)
+      v_write_transposed(qkv, ld, v_off, v_cache, slots, tokens, Hkv, D, page, j / Hkv, j % Hkv,
+                         bias ? bias + (int64_t)(H + Hkv + j % Hkv) * D : nullptr);
     return;
   }
   const bool skip_v = gather_v > 0;
@@ -341,11 +354,20 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
     // the next round's values are on their way while this round is computed
     xv = zero8();
     if (item + per_round < items) xv = *(const bf16x8*)(source(item + per_round) + d0);
+    // (bias: float [q heads | k heads | v heads], a head of D each here: entry item * D + d of any item)
+    float x[8], ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = (float)xc[e];
+    if (bias && live) {
+      const f32x4 b0 = *(const f32x4*)(bias + (int64_t)item * D + d0), b1 = *(const f32x4*)(bias + (int64_t)item * D + d0 + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { x[e] += b0[e]; x[4 + e] += b1[e]; }
+    }
     if (is_v) {
       if (slot >= 0 && !skip_v) {
         bf16* vd = v_cache + ((blk * Hkv + (item - H - Hkv)) * (int64_t)D + d0) * page + off;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) vd[(int64_t)e * page] = xc[e];
+        for (int e = 0; e < 8; ++e) vd[(int64_t)e * page] = (bf16)x[e];
       }
     }
     const bool qk = is_q || is_k;
@@ -365,16 +387,14 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
 #pragma unroll
       for (int e = 0; e < 8; ++e) g[e] = 1.f;
     }
-    float x[8], ss = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      x[e] = (float)xc[e];
-      ss = add_square(ss, x[e]);
-    }
+    for (int e = 0; e < 8; ++e) ss = add_square(ss, x[e]);
     // every lane takes part in the cross-lane steps, whatever its head is
 #pragma unroll
     for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-    const float inv = (qk && w) ? 1.f / sqrtf(ss / (float)D + eps) : 1.f;
+    float inv = (qk && w) ? 1.f / sqrtf(ss / (float)D + eps) : 1.f;
+    // a query grows with its position: 1 + coef ln(floor((p + 1) / every) + 1)
+    if (is_q && w && temp_every > 0) inv *= 1.f + temp_coef * logf((float)((pos[t] + 1) / temp_every) + 1.f);
     float y[8], other[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) y[e] = (qk && w) ? x[e] * inv * g[e] : x[e];
@@ -418,11 +438,12 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES - 1) / WAVES));
   if (temp_every > 0 && !q_gain) return ERR_UNSUPPORTED;
   const bool whole_head_neox = style == 0 && head_dim % 8 == 0 && (!cos_sin || rotary_dim == head_dim) &&
-                               v_dim == head_dim && (v_cache || !slot_mapping) && !bias && temp_every <= 0;
+                               v_dim == head_dim && (v_cache || !slot_mapping);
+  const bool plain_head = !bias && temp_every <= 0;   // what the kernels of 2-byte accesses for whole heads take
   const bool vec_ok = dtype == DT_BF16 && (head_dim == 64 || head_dim == 128 || head_dim == 256) && ld % 8 == 0 &&
                       q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
                       ((uintptr_t)q_gain % 16) == 0 && ((uintptr_t)k_gain % 16) == 0 && ((uintptr_t)cos_sin % 16) == 0 &&
-                      ((uintptr_t)k_cache % 16) == 0;
+                      ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)bias % 16) == 0;
   if (whole_head_neox && vec_ok) {
     const int lph = head_dim / 8, hpw = 64 / lph;
     // many tokens fill the chip with one workgroup each; few tokens spread their heads over several
@@ -435,14 +456,15 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
 #define DINFER_QKV_VEC(LPH_)                                                                                          \
   qkv_post_vec_kernel<LPH_><<<vgrid, WAVES * 64, 0, stream>>>(                                                         \
       (bf16*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps, w_offset, positions, cos_sin, (bf16*)k_cache, \
-      (bf16*)v_cache, slot_mapping, heads, kv_heads, page_size, (int)tokens, (int)gather_v)
+      (bf16*)v_cache, slot_mapping, heads, kv_heads, page_size, (int)tokens, (int)gather_v, bias, temp_coef,       \
+      temp_every)
     if (lph == 8) DINFER_QKV_VEC(8);
     else if (lph == 16) DINFER_QKV_VEC(16);
     else DINFER_QKV_VEC(32);
 #undef DINFER_QKV_VEC
     return launch_status();
   }
-  if (whole_head_neox) {
+  if (whole_head_neox && plain_head) {
     const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES * IPW - 1) / (WAVES * IPW)));
     DINFER_DISPATCH_DTYPE(dtype, {
       if (head_dim <= 128)

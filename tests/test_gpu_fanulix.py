@@ -571,30 +571,78 @@ def test_gated_group_norm_alone(gate_first, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_convolution_with_bias_alone(dtype):
-    """Two requests, one continuing from stored inputs and one starting at position 0 in a slot that held junk."""
+@pytest.mark.parametrize("C,H,K,x0,pad", [(37, 3, 4, 3, 0), (40, 4, 4, 8, 4), (64, 8, 3, 16, 0), (48, 2, 2, 8, 6), (24, 4, 5, 8, 4)])
+def test_convolution_with_bias_alone(C, H, K, x0, pad, dtype):
+    """Two requests, one continuing from stored inputs and one starting at position 0 in a slot that held junk; a
+    third brings one row. Channel counts and offsets that are multiples of 8 run the kernel of 16-byte loads in
+    bfloat16 (2 to 4 taps), the others the kernel of a thread a channel."""
     from dinfer_amd.kernels import ops
     dt = getattr(torch, dtype)
-    C, H, K = 37, 3, 4
     g = torch.Generator().manual_seed(6)
-    full = [torch.randn(n, C + H + 3, generator=g).to(dt) for n in (30, 11)]
+    full = [torch.randn(n, x0 + C + H + pad, generator=g).to(dt) for n in (30, 11, 8)]
     taps, bias = torch.randn(C, K, generator=g) * 0.5, torch.randn(C, generator=g)
     a_log, dt_bias = torch.randn(H, generator=g), torch.randn(H, generator=g)
     conv_state = torch.full((4, C, K - 1), 9.0, dtype=dt, device="cuda")
-    before = 20                                                    # the first request has run 20 tokens already
-    conv_state[2] = full[0][before - (K - 1):before, 3:3 + C].t().cuda()
-    proj = torch.cat([full[0][before:], full[1]]).cuda().contiguous()
-    cu, seq, sl = device_batch([10, 11], [before, 0], [2, 1])
-    work = torch.zeros(21, C + 2 * H, dtype=torch.float32, device="cuda")
-    ops.conv_silu(proj, 21, x_off=3, dt_off=3 + C, taps=taps.cuda(), bias=bias.cuda(), a_log=a_log.cuda(), dt_bias=dt_bias.cuda(),
-                  conv_state=conv_state, state_slots=sl, cu_seqlens=cu, seq_lens=seq, work=work, num_reqs=2)
-    want = [plain.silu(plain.causal_conv(f.double()[:, 3:3 + C], taps.double(), bias.double())) for f in full]
-    want = torch.cat([want[0][before:], want[1]])
+    before, before2 = 20, 7                                        # tokens the first and third request have run already
+    conv_state[2] = full[0][before - (K - 1):before, x0:x0 + C].t().cuda()
+    conv_state[0] = full[2][before2 - (K - 1):before2, x0:x0 + C].t().cuda()
+    rows = torch.cat([full[0][before:], full[1], full[2][before2:]])
+    T = rows.shape[0]
+    cu, seq, sl = device_batch([10, 11, 1], [before, 0, before2], [2, 1, 0])
+    work = torch.zeros(T, C + 2 * H, dtype=torch.float32, device="cuda")
+    ops.conv_silu(rows.cuda().contiguous(), T, x_off=x0, dt_off=x0 + C, taps=taps.cuda(), bias=bias.cuda(), a_log=a_log.cuda(),
+                  dt_bias=dt_bias.cuda(), conv_state=conv_state, state_slots=sl, cu_seqlens=cu, seq_lens=seq, work=work, num_reqs=3)
+    want = [plain.silu(plain.causal_conv(f.double()[:, x0:x0 + C], taps.double(), bias.double())) for f in full]
+    want = torch.cat([want[0][before:], want[1], want[2][before2:]])
     got = work.double().cpu()
     assert (got[:, :C] - want).abs().max().item() < 1e-5 * want.abs().max().item()
-    step = plain.softplus(torch.cat([full[0][before:], full[1]]).double()[:, 3 + C:3 + C + H] + dt_bias.double())
+    step = plain.softplus(rows.double()[:, x0 + C:x0 + C + H] + dt_bias.double())
     assert (got[:, C:C + H] - step).abs().max().item() < 1e-5
     assert (got[:, C + H:] - torch.exp(-torch.exp(a_log.double()) * step)).abs().max().item() < 1e-5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,page,T", [(4, 2, 64, 8, 21), (3, 1, 128, 16, 70), (2, 2, 24, 4, 9)])
+def test_biases_unit_norms_and_temperature_before_the_cache_alone(H, G, D, page, T, dtype):
+    """The step between the joined product and the attention: biases on q, k and v, q and k divided by their root mean
+    square a head, q times its temperature, no rotation; q back in place, k and v into shuffled pages. Heads of 64 and
+    128 run the kernel of 16-byte moves in bfloat16 (70 tokens: its workgroups that gather the values), 24 the plain one."""
+    from dinfer_amd.kernels import ops
+    dt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(D + T)
+    items = H + 2 * G
+    qkv = (torch.randn(T, items * D + 8, generator=g) * 1.5).to(dt)
+    bias = torch.randn(items * D, generator=g) * 2.0
+    coef, every, eps = 0.7, 4, 1e-3
+    start = 13
+    pos = torch.arange(start, start + T, dtype=torch.int32)
+    nb = -(-(start + T) // page)
+    order = list(range(nb + 2))
+    random.Random(T).shuffle(order)
+    slots = torch.tensor([order[p // page] * page + p % page for p in pos.tolist()], dtype=torch.int64)
+    kc = torch.zeros(ops.k_cache_shape(nb + 2, G, page, D), dtype=dt, device="cuda")
+    vc = torch.zeros(ops.v_cache_shape(nb + 2, G, page, D), dtype=dt, device="cuda")
+    buf = qkv.cuda().contiguous()
+    ones = torch.ones(D, dtype=torch.float32, device="cuda")
+    ops.qkv_post(buf, T, heads=H, kv_heads=G, head_dim=D, q_off=8, k_off=8 + H * D, v_off=8 + (H + G) * D, q_gain=ones,
+                 k_gain=ones, eps=eps, gain_offset=0.0, positions=pos.cuda(), cos_sin=None, rotary_dim=0, rope_style=0,
+                 k_cache=kc, v_cache=vc, slot_mapping=slots.cuda(), page_size=page, token_runs=True, bias=bias.cuda(),
+                 q_temp=(coef, every))
+    x = qkv.double()[:, 8:].view(T, items, D) + bias.double().view(items, D)
+    q = plain.rms_unit(x[:, :H], eps) * plain.query_temperature(pos, coef, every).view(T, 1, 1)
+    k, v = plain.rms_unit(x[:, H:H + G], eps), x[:, H + G:]
+    tol = 1e-5 if dtype == "float32" else 1.2e-2
+    assert (buf[:, 8:8 + H * D].double().cpu().view(T, H, D) - q).abs().max().item() < tol * q.abs().max().item()
+    keys = ops.k_cache_rows(kc).double().cpu()[..., :D]          # [blocks, G, page, D]
+    vals = vc.double().cpu().permute(0, 1, 3, 2)                   # [blocks, G, page, D]
+    for i, p in enumerate(pos.tolist()):
+        b, o = order[p // page], p % page
+        assert (keys[b, :, o] - k[i]).abs().max().item() < tol * k.abs().max().item(), f"key of token {i}"
+        assert (vals[b, :, o] - v[i]).abs().max().item() < tol * v.abs().max().item(), f"value of token {i}"
+    used = {order[p // page] for p in pos.tolist()}
+    for b in range(nb + 2):
+        if b not in used:
+            assert (kc[b] == 0).all() and (vc[b] == 0).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
