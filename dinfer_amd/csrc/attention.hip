@@ -931,7 +931,8 @@ int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const b
   // of 512 rows behind 30,000 keys, 352 workgroups instead of 512, loses 17 %). Head size 64 gains nothing.
   constexpr bool WIDE_OK = DT == 8;
   const int64_t wide_blocks = (int64_t)((max_q_len + 47) / 48) * H * num_reqs;
-  if (WIDE_OK && wide_blocks >= 2000) {
+  // (rows of at most two tiles a request never fill the third: many single rows of many heads are no case for it)
+  if (WIDE_OK && max_q_len > 32 && wide_blocks >= 2000) {
     constexpr int QT = WIDE_OK ? 3 : 1;
     const int tiles = (max_q_len + 16 * QT - 1) / (16 * QT);
     if (wide_blocks > 0x7fffffff) return ERR_UNSUPPORTED;

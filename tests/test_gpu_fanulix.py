@@ -45,6 +45,7 @@ P3 = par(6, 1, 8, 16, 1, 32, 48, [0.75], 0, every=1, ls=0.25, rs=2.0)    # no ro
 S3 = ssm(4, 16, 8, 4, 4, 1)                                              # a group a head, four taps
 P4 = par(4, 2, 32, 32, 2, 64, 32, [0.98, 0.999], 32, every=64)           # sizes the matrix-core attention takes
 S4 = ssm(2, 32, 32, 1, 1, 2)                                             # one tap: no convolution state
+P5 = par(4, 1, 64, 64, 3, 16, 24, [0.9, 0.95, 0.99], 16, every=16, coef=0.8)   # heads of 64: 16-byte moves before the cache
 
 CONFIGS = {
     # two streams, pages of 4; a layer without feed-forward, one without a shared expert
@@ -55,6 +56,8 @@ CONFIGS = {
     "F3": (model(80, 48, [moe(S3, 4, 4, 16, 32), moe(P3, 4, 4, 16, 32), moe(S3)], 1, logit_scale=0.5), 16, 13),
     # no `streams`: the plain residual sum; bfloat16: the left attention on the matrix cores (heads of 32, pages of 8)
     "F4": (model(120, 64, [moe(P4, 4, 2, 32, 32), moe(S4, 4, 2, 32, 32), moe(P4)], None, logit_scale=1.3), 8, 14),
+    # three streams; bfloat16: biases, unit norms and temperature in the kernel of 16-byte moves, pages of 16
+    "F5": (model(112, 96, [moe(P5, 8, 3, 24, 48), moe(S1, 8, 3, 24, 48)], 3), 16, 15),
 }
 # one mechanism a model
 ONE = {
@@ -178,7 +181,8 @@ def test_one_mechanism(models, name, dtype):
 def test_which_kernels_and_blocks_serve_which_model(models):
     """bfloat16 with heads and pages the matrix-core kernel takes: that kernel; everything else the plain kernel. A
     model with `streams` runs the streams arrangement on [T, streams * width], one without the plain pre-norm block."""
-    for name, dtype, mfma in (("F4", "bfloat16", True), ("F4", "float32", False), ("F1", "bfloat16", False)):
+    for name, dtype, mfma in (("F4", "bfloat16", True), ("F5", "bfloat16", True), ("F4", "float32", False),
+                              ("F1", "bfloat16", False)):
         r = make_runner(models, name, dtype)
         lefts = [m for b in r.model.blocks if hasattr(b.mixer, "members") for n, m, _, _ in b.mixer.members if n == "left"]
         assert lefts and all(m.mfma_ext == mfma for m in lefts)
