@@ -413,7 +413,9 @@ extern "C" int dinfer_conv_silu(int dtype, const void* proj, int64_t ld, int64_t
   if (tokens <= 0 || num_reqs <= 0) return OK;
   if (C <= 0 || H <= 0 || K <= 0 || tokens > 0x7fffffff || ldw < (int64_t)C + 2 * H) return ERR_BAD_SHAPE;
   if (K > MAX_TAPS) return ERR_UNSUPPORTED;
-  const bool vec = dtype == DT_BF16 && K >= 2 && K <= 4 && C % 8 == 0 && ld % 8 == 0 && x_off % 8 == 0 && ldw % 4 == 0 &&
+  // (single decoded rows take all their earlier inputs from the stored ones, a value at a time: the kernel of a thread
+  // a channel is the faster one there; both add in the same order and give the same bits)
+  const bool vec = tokens >= 4 * (int64_t)num_reqs && dtype == DT_BF16 && K >= 2 && K <= 4 && C % 8 == 0 && ld % 8 == 0 && x_off % 8 == 0 && ldw % 4 == 0 &&
                    ((uintptr_t)proj % 16) == 0 && ((uintptr_t)work % 16) == 0 && ((uintptr_t)taps % 16) == 0 &&
                    ((uintptr_t)bias % 16) == 0;
   if (vec) {
