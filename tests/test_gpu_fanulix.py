@@ -46,6 +46,8 @@ S3 = ssm(4, 16, 8, 4, 4, 1)                                              # a gro
 P4 = par(4, 2, 32, 32, 2, 64, 32, [0.98, 0.999], 32, every=64)           # sizes the matrix-core attention takes
 S4 = ssm(2, 32, 32, 1, 1, 2)                                             # one tap: no convolution state
 P5 = par(4, 1, 64, 64, 3, 16, 24, [0.9, 0.95, 0.99], 16, every=16, coef=0.8)   # heads of 64: 16-byte moves before the cache
+P6 = par(8, 2, 128, 128, 4, 64, 64, [0.9, 0.97, 0.99, 0.999], 32, every=32)    # heads of 128, a quarter of a retention head rotated
+S6 = ssm(8, 32, 64, 2, 4, 4)
 
 CONFIGS = {
     # two streams, pages of 4; a layer without feed-forward, one without a shared expert
@@ -58,6 +60,8 @@ CONFIGS = {
     "F4": (model(120, 64, [moe(P4, 4, 2, 32, 32), moe(S4, 4, 2, 32, 32), moe(P4)], None, logit_scale=1.3), 8, 14),
     # three streams; bfloat16: biases, unit norms and temperature in the kernel of 16-byte moves, pages of 16
     "F5": (model(112, 96, [moe(P5, 8, 3, 24, 48), moe(S1, 8, 3, 24, 48)], 3), 16, 15),
+    # a wider model: heads of 128, sixteen experts
+    "F6": (model(200, 256, [moe(P6, 16, 4, 64, 128), moe(S6, 16, 4, 64, 128), moe(P6, 16, 2, 64, None)], 2, logit_scale=0.8), 16, 23),
 }
 # one mechanism a model
 ONE = {
@@ -181,7 +185,7 @@ def test_one_mechanism(models, name, dtype):
 def test_which_kernels_and_blocks_serve_which_model(models):
     """bfloat16 with heads and pages the matrix-core kernel takes: that kernel; everything else the plain kernel. A
     model with `streams` runs the streams arrangement on [T, streams * width], one without the plain pre-norm block."""
-    for name, dtype, mfma in (("F4", "bfloat16", True), ("F5", "bfloat16", True), ("F4", "float32", False),
+    for name, dtype, mfma in (("F4", "bfloat16", True), ("F5", "bfloat16", True), ("F6", "bfloat16", True), ("F4", "float32", False),
                               ("F1", "bfloat16", False)):
         r = make_runner(models, name, dtype)
         lefts = [m for b in r.model.blocks if hasattr(b.mixer, "members") for n, m, _, _ in b.mixer.members if n == "left"]
@@ -280,6 +284,22 @@ def test_prompt_then_long_decoding(models, name, dtype):
     steps = [([("x", ids[:first], [first - 1])], [])]
     steps += [([("x", [ids[p]], [0])], []) for p in range(first, len(ids))]
     compare_rows(replay(r, steps), cfg, w, {"x": ids}, dtype, f"{name} decode after prompt")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["F2", "F6"])
+def test_a_key_hundreds_of_tokens_back(models, name, dtype):
+    """A prompt of some 700 tokens in two unequal portions, then decoding: every row's softmax runs over hundreds of keys
+    in dozens of pages, the retention's slow heads still carry the first tokens, and the decoded tokens repeat tokens from the
+    prompt's start. (Kernels alone with one far key made to stand out: the recurrence here, the attention where its
+    options were introduced.)"""
+    _, cfg, w, page = models[name]
+    r = make_runner(models, name, dtype, max_tokens=1024, num_blocks=800 // page + 4, max_len=800)
+    ids = tokens_for(cfg, 740, 9)
+    ids[700:] = ids[3:43]                     # decoded tokens repeat tokens 3 .. 42
+    steps = [([("x", ids[:437], [0, 436])], []), ([("x", ids[437:700], [0, 100, 262])], [])]
+    steps += [([("x", [ids[p]], [0])], []) for p in range(700, len(ids))]
+    compare_rows(replay(r, steps), cfg, w, {"x": ids}, dtype, f"{name} far keys")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
