@@ -695,3 +695,72 @@ def test_attention_sink_of_fixed_score_biases_and_temperature(models, dtype):
     # the plain implementation itself: without the sink's one in the denominator the rows would differ
     s = torch.tensor([[-30.0, -31.0]], dtype=F)
     assert plain.softmax_plus_one(s, torch.ones(1, 2, dtype=torch.bool)).sum().item() < 1e-12
+
+
+# ---- the programs a user runs ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_replay_program(models, tmp_path, dtype):
+    """bin/trace_run as a user runs it: a subprocess fed JSON lines; five requests through a pool made for three, so
+    pages and state slots are used again; a request left out of a step; logits read from the files it writes."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    import numpy as np
+    d, cfg, w, page = models["F1"]
+    V = cfg["vocab"]
+    seqs = {k: tokens_for(cfg, n, sum(map(ord, k))) for k, n in (("a", 50), ("b", 90), ("c", 33), ("d", 64), ("e", 20))}
+    plan = [[("a", 30), ("b", 7)], [("a", 20), ("b", 2), ("c", 33)], [("b", 50)], [("b", 1), ("d", 40)],
+            [("b", 1), ("d", 2), ("e", 19)], [("d", 1)], [("b", 29), ("d", 21), ("e", 1)]]
+    steps, fed, expect = [], {k: 0 for k in seqs}, {}
+    for i, st in enumerate(plan):
+        entries, ends = [], []
+        for k, n in st:
+            wants = sorted({0, n - 1})
+            entries.append({"id": k, "tokens": seqs[k][fed[k]:fed[k] + n], "want": wants})
+            expect.setdefault(i, []).extend((k, fed[k] + j) for j in wants)
+            fed[k] += n
+            if fed[k] == len(seqs[k]):
+                ends.append(k)
+        steps.append({"step": i, "entries": entries, "end": ends})
+    assert all(fed[k] == len(v) for k, v in seqs.items())
+    root = Path(__file__).resolve().parent.parent
+    p = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model", str(d), "--dtype", dtype, "--out",
+                        str(tmp_path), "--max-tokens", "256", "--block-size", str(page)],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(plan))]
+    want = {k: plain.forward(cfg, w, v) for k, v in seqs.items()}
+    for i, places in expect.items():
+        got = torch.from_numpy(np.fromfile(tmp_path / f"{i}.f32", dtype="<f4").reshape(len(places), V))
+        check_logits(got.double(), torch.stack([want[k][pos] for k, pos in places]), dtype, f"replayed step {i}")
+
+
+def test_command_line_writes_random_weights_and_generates(models, tmp_path):
+    """bin/dinfer random-weights from a configuration, then bin/dinfer generate on that folder and on a folder of the
+    plain model's weights, where the greedy tokens are the plain model's wherever its choice is clear."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    d, cfg, w, page = models["F2"]
+    root = Path(__file__).resolve().parent.parent
+    exe = [sys.executable, str(root / "bin" / "dinfer")]
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    p = subprocess.run(exe + ["random-weights", "--config", str(tmp_path / "config.json"), "--out", str(tmp_path / "m"), "--seed", "3"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    common = ["--dtype", "float32", "--max-model-len", "128", "--max-num-seqs", "2", "--num-blocks", "64", "--block-size", str(page),
+              "--max-num-batched-tokens", "64", "--max-tokens", "8", "--temperature", "0", "--prompt-ids", "5,9,2", "--prompt-ids", "7"]
+    p = subprocess.run(exe + ["generate", "--model", str(tmp_path / "m")] + common, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    recs = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
+    assert [r["prompt_ids"] for r in recs] == [[5, 9, 2], [7]] and all(len(r["output_ids"]) == 8 for r in recs)
+    p = subprocess.run(exe + ["generate", "--model", str(d)] + common, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    for r in (json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")):
+        ids = list(r["prompt_ids"])
+        for tok in r["output_ids"]:
+            logits = plain.forward(cfg, w, ids)[-1]
+            top2 = logits.topk(2).values
+            if (top2[0] - top2[1]).item() > 1e-3 * logits.std().item():
+                assert tok == int(logits.argmax()), f"greedy token differs after {len(ids)} tokens"
+            ids.append(tok)
