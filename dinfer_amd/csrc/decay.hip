@@ -76,6 +76,59 @@ __global__ void __launch_bounds__(256) rot_widen_kernel(const S* __restrict__ pr
   wr[c] = is_k ? y * k_scale : y;
 }
 
+// The same for bfloat16 rows whose sizes are multiples of 8 (half the rotated entries too): a thread takes 8 consecutive
+// entries of a head, so they lie wholly in the first half of the rotated entries, in the second, or behind them; its
+// values, its partners' and the angles come as 16- and 32-byte loads and the floats leave as two 16-byte stores.
+__global__ void __launch_bounds__(256) rot_widen_vec_kernel(const bf16* __restrict__ proj, int64_t ld, int64_t q_off,
+                                                            int64_t k_off, int64_t v_off, const int32_t* __restrict__ pos,
+                                                            const float* __restrict__ cos_sin, int rot, float k_scale,
+                                                            float* __restrict__ work, int64_t ldw, int H, int D, int V) {
+  const int64_t t = blockIdx.x;
+  const bf16* row = proj + t * ld;
+  float* wr = work + t * ldw;
+  const int half = rot / 2;
+  const int hd = H * D;
+  const int c = 8 * (blockIdx.y * 256 + threadIdx.x);
+  if (c >= 2 * hd + H * V) return;
+  float y[8];
+  if (c >= 2 * hd) {
+    const bf16x8 v = *(const bf16x8*)(row + v_off + c - 2 * hd);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = (float)v[e];
+  } else {
+    const bool is_k = c >= hd;
+    const int e0 = is_k ? c - hd : c;
+    const int d = e0 % D;
+    const bf16* src = row + (is_k ? k_off : q_off);
+    const bf16x8 v = *(const bf16x8*)(src + e0);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = (float)v[e];
+    if (cos_sin && d < rot) {
+      const float* cs = cos_sin + (int64_t)pos[t] * rot;
+      const bool first = d < half;
+      const int i = first ? d : d - half;
+      const bf16x8 o = *(const bf16x8*)(src + (first ? e0 + half : e0 - half));
+      const f32x4 c0 = *(const f32x4*)(cs + i), c1 = *(const f32x4*)(cs + i + 4);
+      const f32x4 s0 = *(const f32x4*)(cs + half + i), s1 = *(const f32x4*)(cs + half + i + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float cc = e < 4 ? c0[e & 3] : c1[e & 3], sn = e < 4 ? s0[e & 3] : s1[e & 3];
+        const float other = (float)o[e];
+        y[e] = first ? rotated_first(y[e], other, cc, sn) : rotated_second(other, y[e], cc, sn);
+      }
+    }
+    if (is_k) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] *= k_scale;
+    }
+  }
+  f32x4 a, b;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { a[e] = y[e]; b[e] = y[4 + e]; }
+  *(f32x4*)(wr + c) = a;
+  *(f32x4*)(wr + c + 4) = b;
+}
+
 // work row: the C channels after convolution, bias and silu | dt (H) | decay (H), float
 template <class S>
 __global__ void __launch_bounds__(256) conv_silu_kernel(
@@ -382,6 +435,49 @@ __global__ void __launch_bounds__(256) gated_group_norm_kernel(const float* __re
   }
 }
 
+// The same for groups of up to 256 columns: a wave a (token, group), a lane up to 4 of its columns, the sum of squares by
+// shuffles; no LDS and no barrier (a retention's groups are its heads: 128 columns were half a workgroup idle).
+template <class S>
+__global__ void __launch_bounds__(256) gated_group_norm_wave_kernel(const float* __restrict__ y, int64_t ld_y,
+                                                                    const float* __restrict__ x, int64_t ld_x,
+                                                                    const float* __restrict__ skip, int V,
+                                                                    const S* __restrict__ z, int64_t ld_z, int64_t z_off,
+                                                                    const float* __restrict__ w, S* __restrict__ out,
+                                                                    int64_t ld_out, int64_t col_off, int groups, int group,
+                                                                    float eps, float out_scale, int gate_first) {
+  const int64_t t = blockIdx.x;
+  const int g = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (g >= groups) return;                   // (a whole wave leaves: the shuffles below see full waves only)
+  const int c0 = g * group;
+  float kept[4], gate[4];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int i = lane + 64 * e;
+    kept[e] = 0.f;
+    gate[e] = 0.f;
+    if (i < group) {
+      const int c = c0 + i;
+      float u = y[t * ld_y + c];
+      if (skip) u = __builtin_fmaf(skip[c / V], x[t * ld_x + c], u);
+      gate[e] = silu_f(to_f32(z[t * ld_z + z_off + c]));
+      kept[e] = gate_first ? u * gate[e] : u;
+    }
+    ss = __builtin_fmaf(kept[e], kept[e], ss);
+  }
+  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)group + eps);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int i = lane + 64 * e;
+    if (i < group) {
+      const int c = c0 + i;
+      float r = kept[e] * inv * (w ? w[c] : 1.f) * out_scale;
+      if (!gate_first) r *= gate[e];
+      out[t * ld_out + col_off + c] = from_f32<S>(r);
+    }
+  }
+}
+
 }  // namespace
 
 // proj [T, ld] in the step's dtype: H heads of q (size D) from column q_off, of k from k_off, H heads of v (size V) from
@@ -394,6 +490,16 @@ extern "C" int dinfer_rot_widen(int dtype, const void* proj, int64_t ld, int64_t
   if (H <= 0 || D <= 0 || V <= 0 || rot < 0 || rot > D || rot % 2 || tokens > 0x7fffffff ||
       ldw < 2 * (int64_t)H * D + (int64_t)H * V)
     return ERR_BAD_SHAPE;
+  const bool vec = dtype == DT_BF16 && D % 8 == 0 && V % 8 == 0 && (!cos_sin || rot % 16 == 0) && ld % 8 == 0 &&
+                   q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && ldw % 4 == 0 && ((uintptr_t)proj % 16) == 0 &&
+                   ((uintptr_t)work % 16) == 0 && ((uintptr_t)cos_sin % 16) == 0;
+  if (vec) {
+    const int pieces = (2 * H * D + H * V) / 8;
+    const dim3 vgrid((unsigned)tokens, (unsigned)((pieces + 255) / 256));
+    rot_widen_vec_kernel<<<vgrid, 256, 0, stream>>>((const bf16*)proj, ld, q_off, k_off, v_off, positions, cos_sin, rot,
+                                                    k_scale, work, ldw, H, D, V);
+    return launch_status();
+  }
   const dim3 grid((unsigned)tokens, (unsigned)((2 * H * D + H * V + 255) / 256));
   DINFER_DISPATCH_DTYPE(dtype, {
     rot_widen_kernel<S><<<grid, 256, 0, stream>>>((const S*)proj, ld, q_off, k_off, v_off, positions, cos_sin,
@@ -470,6 +576,15 @@ extern "C" int dinfer_gated_group_norm(int dtype, const float* y, int64_t ld_y, 
                                        hipStream_t stream) {
   if (tokens <= 0) return OK;
   if (groups <= 0 || group <= 0 || groups > 65535 || tokens > 0x7fffffff || (skip && (!x || V <= 0))) return ERR_BAD_SHAPE;
+  if (group <= 256) {
+    const dim3 wgrid((unsigned)tokens, (unsigned)((groups + 3) / 4));
+    DINFER_DISPATCH_DTYPE(dtype, {
+      gated_group_norm_wave_kernel<S><<<wgrid, 256, 0, stream>>>(y, ld_y, x, ld_x, skip, V, (const S*)z, ld_z, z_off, w,
+                                                                (S*)out, ld_out, col_off, groups, group, eps, out_scale,
+                                                                gate_first);
+    });
+    return launch_status();
+  }
   const dim3 grid((unsigned)tokens, (unsigned)groups);
   DINFER_DISPATCH_DTYPE(dtype, {
     gated_group_norm_kernel<S><<<grid, 256, 0, stream>>>(y, ld_y, x, ld_x, skip, V, (const S*)z, ld_z, z_off, w, (S*)out,

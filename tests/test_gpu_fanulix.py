@@ -532,22 +532,25 @@ def test_decay_recurrence_alone(case):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_rotation_of_half_pairs_alone(dtype):
+@pytest.mark.parametrize("H,D,V,rot,off", [(3, 20, 12, 12, 5), (3, 32, 24, 16, 8), (2, 64, 40, 64, 16), (4, 16, 8, 0, 8)])
+def test_rotation_of_half_pairs_alone(H, D, V, rot, off, dtype):
+    """Sizes that are multiples of 8 with half the rotated entries a multiple of 8 run the kernel of 8 entries a thread in
+    bfloat16 (part of a head rotated, a whole head, none), the others the kernel of a thread an entry."""
     from dinfer_amd.kernels import ops
     from dinfer_amd.parts.position import Rotary
     dt = getattr(torch, dtype)
-    H, D, V, rot, T = 3, 20, 12, 12, 50
+    T = 50
     g = torch.Generator().manual_seed(2)
-    proj = torch.randn(T, 2 * H * D + H * V + 5, generator=g).to(dt)
+    proj = torch.randn(T, -(-(2 * H * D + H * V + off) // 8) * 8, generator=g).to(dt)
     pos = torch.randint(0, 3000, (T,), generator=g, dtype=torch.int32)
-    table = Rotary(head_dim=D, theta=700.0, max_positions=4096, rotary_dim=rot).host_table(4096).cuda()
+    table = Rotary(head_dim=D, theta=700.0, max_positions=4096, rotary_dim=rot).host_table(4096).cuda() if rot else None
     work = torch.zeros(T, 2 * H * D + H * V, dtype=torch.float32, device="cuda")
-    ops.rot_widen(proj.cuda(), T, q_off=5, k_off=5 + H * D, v_off=5 + 2 * H * D, positions=pos.cuda(), cos_sin=table,
+    ops.rot_widen(proj.cuda(), T, q_off=off, k_off=off + H * D, v_off=off + 2 * H * D, positions=pos.cuda(), cos_sin=table,
                   rotary_dim=rot, k_scale=0.37, work=work, heads=H, dim=D, vdim=V)
     x = proj.double()
-    q = plain.rotate_half(x[:, 5:5 + H * D].view(T, H, D), pos, 700.0, rot).reshape(T, -1)
-    k = plain.rotate_half(x[:, 5 + H * D:5 + 2 * H * D].view(T, H, D), pos, 700.0, rot).reshape(T, -1) * 0.37
-    want = torch.cat([q, k, x[:, 5 + 2 * H * D:]], dim=1)
+    q = plain.rotate_half(x[:, off:off + H * D].view(T, H, D), pos, 700.0, rot).reshape(T, -1)
+    k = plain.rotate_half(x[:, off + H * D:off + 2 * H * D].view(T, H, D), pos, 700.0, rot).reshape(T, -1) * 0.37
+    want = torch.cat([q, k, x[:, off + 2 * H * D:off + 2 * H * D + H * V]], dim=1)
     assert (work.double().cpu() - want).abs().max().item() < 3e-4      # (angles of a few thousand radians in 32 bits)
 
 
@@ -589,10 +592,13 @@ def test_streams_step_alone(n, width, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("gate_first", [True, False])
-def test_gated_group_norm_alone(gate_first, dtype):
+@pytest.mark.parametrize("H,V,groups", [(6, 20, 3), (6, 20, 6), (5, 128, 5), (8, 80, 2), (16, 80, 1)])
+def test_gated_group_norm_alone(H, V, groups, gate_first, dtype):
+    """Groups of 40, 20 and 128 columns (a wave a group; five groups: a workgroup's last waves idle), of 320 (a workgroup
+    a group, kept in registers) and of 1,280 (read twice)."""
     from dinfer_amd.kernels import ops
     dt = getattr(torch, dtype)
-    T, H, V, groups = 7, 6, 20, 3
+    T = 7
     n = H * V
     g = torch.Generator().manual_seed(4)
     y, x = torch.randn(T, n, generator=g), torch.randn(T, n, generator=g)
