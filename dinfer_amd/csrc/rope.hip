@@ -345,6 +345,13 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
   const int wave_first = (blockIdx.y * WAVES + wave) * HPW;
   bf16x8 xv = zero8();
   if (first_item < items) xv = *(const bf16x8*)(source(first_item) + d0);
+  // (bias: float [q heads | k heads | v heads], a head of D each here: entry item * D + d of any item; asked for with the
+  // values it is added to, a round ahead)
+  f32x4 bn0 = {0.f, 0.f, 0.f, 0.f}, bn1 = {0.f, 0.f, 0.f, 0.f};
+  if (bias && first_item < items) {
+    bn0 = *(const f32x4*)(bias + (int64_t)first_item * D + d0);
+    bn1 = *(const f32x4*)(bias + (int64_t)first_item * D + d0 + 4);
+  }
   for (int base = 0; wave_first + base < items; base += per_round) {
     const int item = first_item + base;
     const bool live = item < items;
@@ -353,13 +360,18 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
     const bf16x8 xc = xv;
     // the next round's values are on their way while this round is computed
     xv = zero8();
-    if (item + per_round < items) xv = *(const bf16x8*)(source(item + per_round) + d0);
-    // (bias: float [q heads | k heads | v heads], a head of D each here: entry item * D + d of any item)
+    const f32x4 b0 = bn0, b1 = bn1;
+    if (item + per_round < items) {
+      xv = *(const bf16x8*)(source(item + per_round) + d0);
+      if (bias) {
+        bn0 = *(const f32x4*)(bias + (int64_t)(item + per_round) * D + d0);
+        bn1 = *(const f32x4*)(bias + (int64_t)(item + per_round) * D + d0 + 4);
+      }
+    }
     float x[8], ss = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) x[e] = (float)xc[e];
     if (bias && live) {
-      const f32x4 b0 = *(const f32x4*)(bias + (int64_t)item * D + d0), b1 = *(const f32x4*)(bias + (int64_t)item * D + d0 + 4);
 #pragma unroll
       for (int e = 0; e < 4; ++e) { x[e] += b0[e]; x[4 + e] += b1[e]; }
     }
