@@ -74,4 +74,8 @@ def load_config(model_dir: str | Path) -> tuple[Architecture, ModelConfig]:
     except json.JSONDecodeError as e:
         raise ConfigError(f"{path} is not valid JSON: {e}") from e
     arch = architecture_of(d)
+    fill = getattr(arch.config_class, "sizes_from_tensors", None)
+    if fill is not None:      # a design some of whose sizes only a tensor's shape gives
+        from ..weights.safetensors_io import tensor_shapes
+        d = fill(d, tensor_shapes(model_dir))
     return arch, arch.config_class.from_dict(d)

@@ -134,6 +134,115 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
   }
 }
 
+// Differential attention: a query head holds two queries of D entries, [first map | second map], and so does a key
+// head; each map is a softmax attention of its own over the same values, and the head's output is
+//   o = a1 - lambda a2,   o <- o / sqrt(mean(o^2) + eps) * post      (the mean over the head's Dv values)
+// One wave per (token, query head) walks the keys once and keeps both maps' (max, sum, output). The key pages hold
+// heads of 2 D entries, the value pages heads of Dv.
+template <class S>
+__global__ void __launch_bounds__(WAVES * 64) attn_paged_diff_kernel(
+    const S* __restrict__ q, int64_t ld_q, S* __restrict__ out, int64_t ld_out, const S* __restrict__ k_cache,
+    const S* __restrict__ v_cache, const int32_t* __restrict__ block_table, int64_t max_blocks,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int num_reqs, float scale,
+    int window, int H, int Hkv, int D, int page, int Dv, float lambda, float eps, float post) {
+  __shared__ float qs[WAVES][MAX_D];
+  __shared__ float ps[WAVES][2][64];
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * WAVES + wave;
+  const bool live = h < H;
+
+  int lo_b = 0, hi_b = num_reqs - 1;
+  while (lo_b < hi_b) {
+    const int mid = (lo_b + hi_b + 1) >> 1;
+    if (cu_seqlens[mid] <= t) lo_b = mid; else hi_b = mid - 1;
+  }
+  const int b = lo_b;
+  const int q_len = cu_seqlens[b + 1] - cu_seqlens[b];
+  const int p = seq_lens[b] - q_len + (t - cu_seqlens[b]);
+  const int first_key = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+  const int32_t* bt = block_table + (int64_t)b * max_blocks;
+  const int hk = live ? h / (H / Hkv) : 0;
+  const int D2 = 2 * D;
+  const int Dp = (D2 + 7) & ~7;
+
+  if (live) {
+    const S* qr = q + (int64_t)t * ld_q + (int64_t)h * D2;
+    for (int d = lane; d < D2; d += 64) qs[wave][d] = to_f32(qr[d]);
+  }
+  __syncthreads();
+
+  constexpr int NC = MAX_D / 64;
+  float o1[NC], o2[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) o1[c] = o2[c] = 0.f;
+  float m1 = -INFINITY, l1 = 0.f, m2 = -INFINITY, l2 = 0.f;
+
+  for (int j0 = first_key; j0 <= p; j0 += 64) {
+    const int j = j0 + lane;
+    float s1 = -INFINITY, s2 = -INFINITY;
+    if (live && j <= p) {
+      const int blk = bt[j / page];
+      const S* kr = k_cache + ((int64_t)blk * Hkv + hk) * page * Dp;
+      const int off = j % page;
+      float acc1 = 0.f, acc2 = 0.f;
+      for (int d = 0; d < D; ++d) {
+        acc1 += qs[wave][d] * to_f32(kr[k_page_offset(off, d, page)]);
+        acc2 += qs[wave][D + d] * to_f32(kr[k_page_offset(off, D + d, page)]);
+      }
+      s1 = acc1 * scale;
+      s2 = acc2 * scale;
+    }
+    const float n1 = fmaxf(m1, wave_max(s1)), n2 = fmaxf(m2, wave_max(s2));
+    const float p1 = (live && j <= p) ? expf(s1 - n1) : 0.f, p2 = (live && j <= p) ? expf(s2 - n2) : 0.f;
+    const float al1 = expf(m1 - n1), al2 = expf(m2 - n2);
+    l1 = l1 * al1 + wave_sum(p1);
+    l2 = l2 * al2 + wave_sum(p2);
+    m1 = n1;
+    m2 = n2;
+    __syncthreads();
+    ps[wave][0][lane] = p1;
+    ps[wave][1][lane] = p2;
+    __syncthreads();
+    if (live) {
+      const int n = p - j0 + 1 < 64 ? p - j0 + 1 : 64;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int d = lane + 64 * c;
+        if (d < Dv) {
+          float x1 = o1[c] * al1, x2 = o2[c] * al2;
+          for (int jj = 0; jj < n; ++jj) {
+            const int key = j0 + jj;
+            const int blk = bt[key / page];
+            const float v = to_f32(v_cache[(((int64_t)blk * Hkv + hk) * Dv + d) * page + (key % page)]);
+            x1 += ps[wave][0][jj] * v;
+            x2 += ps[wave][1][jj] * v;
+          }
+          o1[c] = x1;
+          o2[c] = x2;
+        }
+      }
+    }
+  }
+  if (live) {
+    const float i1 = l1 > 0.f ? 1.f / l1 : 0.f, i2 = l2 > 0.f ? lambda / l2 : 0.f;
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int d = lane + 64 * c;
+      o1[c] = d < Dv ? o1[c] * i1 - o2[c] * i2 : 0.f;
+      ss += o1[c] * o1[c];
+    }
+    const float inv = post / sqrtf(wave_sum(ss) / (float)Dv + eps);
+    S* orow = out + (int64_t)t * ld_out + (int64_t)h * Dv;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int d = lane + 64 * c;
+      if (d < Dv) orow[d] = from_f32<S>(o1[c] * inv);
+    }
+  }
+}
+
 }  // namespace
 
 // q [T, ld_q] (head h at column h*D), out [T, ld_out]; block_table [num_reqs, max_blocks];
@@ -177,6 +286,28 @@ extern "C" int dinfer_attn_paged_ext(int dtype, const void* q, int64_t ld_q, voi
         (const S*)q, ld_q, (S*)out, ld_out, (const S*)k_cache, (const S*)v_cache, block_table, max_blocks, cu_seqlens,
         seq_lens, num_reqs, scale, window, heads, kv_heads, head_dim, page_size, window > 0 ? keep_first : 0, sinks,
         slope_exp, v_dim, out_scale);
+  });
+  return launch_status();
+}
+
+// Differential attention (see the kernel). q [T, ld_q]: head h at column 2 h head_dim, first map then second; the key
+// pages hold kv_heads heads of 2 head_dim entries, the value pages heads of v_dim; out [T, ld_out], head h at h v_dim.
+extern "C" int dinfer_attn_paged_diff(int dtype, const void* q, int64_t ld_q, void* out, int64_t ld_out,
+                                      const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                      int64_t max_blocks, const int32_t* cu_seqlens, const int32_t* seq_lens,
+                                      int num_reqs, int64_t tokens, float scale, int window, int heads, int kv_heads,
+                                      int head_dim, int v_dim, int page_size, float lambda, float eps, float post,
+                                      hipStream_t stream) {
+  if (tokens <= 0 || num_reqs <= 0) return OK;
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim <= 0 || v_dim <= 0 || page_size <= 0 ||
+      max_blocks <= 0 || window < 0 || tokens > 0x7fffffff || !v_cache)
+    return ERR_BAD_SHAPE;
+  if (2 * head_dim > MAX_D || v_dim > MAX_D) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tokens, (unsigned)((heads + WAVES - 1) / WAVES));
+  DINFER_DISPATCH_DTYPE(dtype, {
+    attn_paged_diff_kernel<S><<<grid, WAVES * 64, 0, stream>>>(
+        (const S*)q, ld_q, (S*)out, ld_out, (const S*)k_cache, (const S*)v_cache, block_table, max_blocks, cu_seqlens,
+        seq_lens, num_reqs, scale, window, heads, kv_heads, head_dim, page_size, v_dim, lambda, eps, post);
   });
   return launch_status();
 }

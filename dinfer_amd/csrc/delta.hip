@@ -351,7 +351,7 @@ __global__ void __launch_bounds__(WAVES * 64) delta_out_kernel(const float* __re
                                                                const S* __restrict__ proj, int64_t ld, int64_t g_off,
                                                                const float* __restrict__ w, S* __restrict__ out,
                                                                int64_t ld_out, int64_t col_off, int H, int V, float eps,
-                                                               float out_scale) {
+                                                               float out_scale, int w_stride, int gate_kind) {
   const int t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int h = blockIdx.y * WAVES + wave;
@@ -370,9 +370,180 @@ __global__ void __launch_bounds__(WAVES * 64) delta_out_kernel(const float* __re
   for (int e = 0; e < PER; ++e) {
     const int d = lane + 64 * e;
     if (d < V) {
-      const float gate = silu_f(to_f32(proj[(int64_t)t * ld + g_off + h * V + d]));
-      out[(int64_t)t * ld_out + col_off + h * V + d] = from_f32<S>(x[e] * inv * w[d] * gate * out_scale);
+      const float gl = to_f32(proj[(int64_t)t * ld + g_off + h * V + d]);
+      const float gate = gate_kind == 1 ? sigmoid_f(gl) : silu_f(gl);
+      out[(int64_t)t * ld_out + col_off + h * V + d] = from_f32<S>(x[e] * inv * w[h * w_stride + d] * gate * out_scale);
     }
+  }
+}
+
+
+// ---- delta rule with a decay and a removal rate of its own for every key channel ------------------------------------
+//
+//   per token, per head:   S <- diag(w) S - (a * u) (u^T S) + k v^T   (both terms from the state before);   o = S^T r
+//
+// u = k / sqrt(sum k^2 + eps) the unit key, w in (0, 1) a decay and a in (0, 1) a removal rate a key channel. Column j
+// of S goes its own way: s' = w * s - (a * u) A + k v_j with A = u . s, and o_j = r . s' = (r * w) . s - c1 A + c2 v_j
+// with c1 = r . (a * u) and c2 = r . k, which depend on the token alone. So a token costs a column two sums (A and
+// (r * w) . s), taken at once from the state before, and nothing waits for the update.
+//
+//   channel_delta_prep        one wave a (token, head): unit key, removal rate, decay
+//                             w = exp(-rate * sigmoid(W2 tanh(l) + w0)) from the low-rank projection l, c1, c2. Float out.
+//   channel_delta_recurrence  the layout of delta_recurrence: a request, a head and COLS columns a workgroup, 32 lanes a
+//                             column, CH tokens' operands waiting in LDS while the next CH are on their way.
+constexpr int MAX_LOW = 512;   // the largest inner size of the decay's low-rank projection
+
+// work [T, ldw] float: rw (H D) | u (H D) | k (H D) | w (H D) | au (H D) | v (H D) | c1 (H) | c2 (H)
+template <class S>
+__global__ void __launch_bounds__(WAVES * 64) channel_delta_prep_kernel(
+    const S* __restrict__ proj, int64_t ld, int64_t r_off, int64_t k_off, int64_t v_off, int64_t a_off, int64_t l_off,
+    const float* __restrict__ a_bias, const float* __restrict__ w2, const float* __restrict__ w0, int low,
+    float* __restrict__ work, int64_t ldw, int H, int D, float eps, float rate) {
+  __shared__ float th[WAVES][MAX_LOW];
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * WAVES + wave;
+  if (h >= H) return;   // (no workgroup barrier below)
+  const S* row = proj + (int64_t)t * ld;
+  float* out = work + (int64_t)t * ldw;
+  const int HD = H * D;
+  for (int l = lane; l < low; l += 64) th[wave][l] = tanhf(to_f32(row[l_off + l]));
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  constexpr int PER = MAX_HEAD / 64;
+  float kk[PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int d = lane + 64 * e;
+    kk[e] = d < D ? to_f32(row[k_off + h * D + d]) : 0.f;
+    ss = __builtin_fmaf(kk[e], kk[e], ss);
+  }
+  const float inv = 1.f / sqrtf(wave_sum(ss) + eps);
+  float c1 = 0.f, c2 = 0.f;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int d = lane + 64 * e;
+    if (d < D) {
+      const int c = h * D + d;
+      const float r = to_f32(row[r_off + c]);
+      const float u = kk[e] * inv;
+      const float a = sigmoid_f(to_f32(row[a_off + c]) + a_bias[c]);
+      float z = w0[c];
+      const float* w2r = w2 + (int64_t)c * low;
+      for (int l = 0; l < low; ++l) z = __builtin_fmaf(w2r[l], th[wave][l], z);
+      const float w = expf(-rate * sigmoid_f(z));
+      const float au = a * u;
+      out[c] = r * w;
+      out[HD + c] = u;
+      out[2 * HD + c] = kk[e];
+      out[3 * HD + c] = w;
+      out[4 * HD + c] = au;
+      out[5 * HD + c] = to_f32(row[v_off + c]);
+      c1 = __builtin_fmaf(r, au, c1);
+      c2 = __builtin_fmaf(r, kk[e], c2);
+    }
+  }
+  c1 = wave_sum(c1);
+  c2 = wave_sum(c2);
+  if (lane == 0) {
+    out[6 * HD + h] = c1;
+    out[6 * HD + H + h] = c2;
+  }
+}
+
+template <int RPT, int CHT>
+__global__ void __launch_bounds__(256) channel_delta_recurrence_kernel(
+    const float* __restrict__ work, int64_t ldw, float* __restrict__ state, const int32_t* __restrict__ slots,
+    const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_lens, float* __restrict__ out, int64_t ld_out,
+    int H, int D) {
+  constexpr int DP = 32 * RPT;
+  constexpr int NV = 5;   // rw, u, k, w, au
+  __shared__ __attribute__((aligned(16))) float vec[NV][CHT][DP];
+  __shared__ float vs[CHT][COLS];
+  __shared__ float cs[2][CHT];
+  const int b = blockIdx.z, h = blockIdx.y, cb = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int rg = tid & 31, cj = tid >> 5;
+  const int j = cb * COLS + cj;
+  const int t0 = cu[b], n = cu[b + 1] - t0;
+  const int start = seq_lens[b] - n;
+  const int HD = H * D;
+  const bool col_ok = j < D;
+  float* sp = state + ((((int64_t)slots[b] * H + h) * D + (col_ok ? j : 0)) * D) + rg * RPT;
+  float S[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) S[i] = (start > 0 && col_ok && rg * RPT + i < D) ? sp[i] : 0.f;
+
+  constexpr int PK = (CHT * DP) / 256;
+  static_assert(PK >= 1 && (CHT * DP) % 256 == 0, "a chunk's vectors are dealt evenly among the threads");
+  float pre[NV][PK], pv = 0.f, pc = 0.f;
+  const float* wk = work + (int64_t)t0 * ldw;
+  auto fetch = [&](int ct) {
+#pragma unroll
+    for (int e = 0; e < PK; ++e) {
+      const int idx = tid + e * 256;
+      const int tok = idx / DP, d = idx % DP;
+      const bool ok = ct + tok < n && d < D;
+      const float* r = wk + (int64_t)(ct + tok) * ldw + h * D + d;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) pre[v][e] = ok ? r[v * HD] : 0.f;
+    }
+    if (tid < CHT * COLS) {
+      const int tok = tid / COLS, c = tid % COLS;
+      const int col = cb * COLS + c;
+      pv = (ct + tok < n && col < D) ? wk[(int64_t)(ct + tok) * ldw + 5 * HD + h * D + col] : 0.f;
+    }
+    if (tid < 2 * CHT) {
+      const int tok = tid % CHT;
+      pc = ct + tok < n ? wk[(int64_t)(ct + tok) * ldw + 6 * HD + (tid < CHT ? 0 : H) + h] : 0.f;
+    }
+  };
+  fetch(0);
+  for (int ct = 0; ct < n; ct += CHT) {
+    __syncthreads();  // the chunk before has been consumed
+#pragma unroll
+    for (int e = 0; e < PK; ++e) {
+      const int idx = tid + e * 256;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) vec[v][idx / DP][idx % DP] = pre[v][e];
+    }
+    if (tid < CHT * COLS) vs[tid / COLS][tid % COLS] = pv;
+    if (tid < 2 * CHT) cs[tid / CHT][tid % CHT] = pc;
+    __syncthreads();
+    if (ct + CHT < n) fetch(ct + CHT);  // in flight while this chunk is worked through
+    const int m = n - ct < CHT ? n - ct : CHT;
+    for (int tok = 0; tok < m; ++tok) {
+      float rw[RPT], u[RPT];
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        rw[i] = vec[0][tok][rg * RPT + i];
+        u[i] = vec[1][tok][rg * RPT + i];
+      }
+      float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;   // two chains a sum: a fixed order all the same
+#pragma unroll
+      for (int i = 0; i < RPT; i += 2) {
+        a0 = __builtin_fmaf(S[i], u[i], a0);
+        b0 = __builtin_fmaf(S[i], rw[i], b0);
+        if (i + 1 < RPT) {
+          a1 = __builtin_fmaf(S[i + 1], u[i + 1], a1);
+          b1 = __builtin_fmaf(S[i + 1], rw[i + 1], b1);
+        }
+      }
+      const float vt = vs[tok][cj], c1 = cs[0][tok], c2 = cs[1][tok];
+      const float A = half_wave_sum(a0 + a1), B = half_wave_sum(b0 + b1);
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        const float k = vec[2][tok][rg * RPT + i], w = vec[3][tok][rg * RPT + i], au = vec[4][tok][rg * RPT + i];
+        S[i] = __builtin_fmaf(k, vt, __builtin_fmaf(-au, A, w * S[i]));
+      }
+      if (rg == 0 && col_ok) out[(int64_t)(t0 + ct + tok) * ld_out + h * D + j] = __builtin_fmaf(c2, vt, __builtin_fmaf(-c1, A, B));
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+      if (rg * RPT + i < D) sp[i] = S[i];
   }
 }
 
@@ -447,16 +618,55 @@ extern "C" int dinfer_delta_recurrence(const float* work, int64_t ldw, float* st
 }
 
 // out[t, col_off + h V + d] = o[t, h V + d] / sqrt(mean_d o^2 + eps) * w[d] * silu(proj[t, g_off + h V + d]) * out_scale
+// w_per_head: w holds H V gains, a head's own at h V; gate_kind: 0 silu, 1 the logistic function.
 extern "C" int dinfer_delta_out(int dtype, const float* o, int64_t ld_o, const void* proj, int64_t ld, int64_t g_off,
                                 const float* w, void* out, int64_t ld_out, int64_t col_off, int64_t tokens, int H, int V,
-                                float eps, float out_scale, hipStream_t stream) {
+                                float eps, float out_scale, int w_per_head, int gate_kind, hipStream_t stream) {
+  if (gate_kind != 0 && gate_kind != 1) return ERR_UNSUPPORTED;
   if (tokens <= 0) return OK;
   if (H <= 0 || V <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
   if (V > MAX_HEAD) return ERR_UNSUPPORTED;
   const dim3 grid((unsigned)tokens, (unsigned)((H + WAVES - 1) / WAVES));
   DINFER_DISPATCH_DTYPE(dtype, {
     delta_out_kernel<S><<<grid, WAVES * 64, 0, stream>>>(o, ld_o, (const S*)proj, ld, g_off, w, (S*)out, ld_out,
-                                                         col_off, H, V, eps, out_scale);
+                                                         col_off, H, V, eps, out_scale, w_per_head ? V : 0, gate_kind);
   });
+  return launch_status();
+}
+
+// The rule with a decay and a removal rate a key channel (see above). proj [T, ld]: r, k, v (H D each) at their columns,
+// the H D removal logits at a_off, the `low` entries of the decay's inner projection at l_off. a_bias, w0 [H D] float,
+// w2 [H D, low] float. work [T, ldw] float, ldw >= 6 H D + 2 H.
+extern "C" int dinfer_channel_delta_prep(int dtype, const void* proj, int64_t ld, int64_t r_off, int64_t k_off,
+                                         int64_t v_off, int64_t a_off, int64_t l_off, const float* a_bias,
+                                         const float* w2, const float* w0, int low, float* work, int64_t ldw,
+                                         int64_t tokens, int H, int D, float eps, float rate, hipStream_t stream) {
+  if (tokens <= 0) return OK;
+  if (H <= 0 || D <= 0 || low <= 0 || tokens > 0x7fffffff || ldw < 6LL * H * D + 2 * H) return ERR_BAD_SHAPE;
+  if (D > MAX_HEAD || low > MAX_LOW) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tokens, (unsigned)((H + WAVES - 1) / WAVES));
+  DINFER_DISPATCH_DTYPE(dtype, {
+    channel_delta_prep_kernel<S><<<grid, WAVES * 64, 0, stream>>>((const S*)proj, ld, r_off, k_off, v_off, a_off, l_off,
+                                                                  a_bias, w2, w0, low, work, ldw, H, D, eps, rate);
+  });
+  return launch_status();
+}
+
+// state [slots, H, D, D] float (a head's matrix transposed: [value, key]); out [T, ld_out] float, head h at h D.
+extern "C" int dinfer_channel_delta_recurrence(const float* work, int64_t ldw, float* state, const int32_t* state_slots,
+                                               const int32_t* cu_seqlens, const int32_t* seq_lens, float* out,
+                                               int64_t ld_out, int num_reqs, int H, int D, hipStream_t stream) {
+  if (num_reqs <= 0) return OK;
+  if (H <= 0 || D <= 0 || num_reqs > 65535 || H > 65535) return ERR_BAD_SHAPE;
+  if (D > 256) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)((D + COLS - 1) / COLS), (unsigned)H, (unsigned)num_reqs);
+#define CHANNEL_REC(R_, C_)                                                                                          \
+  channel_delta_recurrence_kernel<R_, C_><<<grid, 256, 0, stream>>>(work, ldw, state, state_slots, cu_seqlens,       \
+                                                                    seq_lens, out, ld_out, H, D)
+  if (D <= 32) CHANNEL_REC(1, 16);
+  else if (D <= 64) CHANNEL_REC(2, 16);
+  else if (D <= 128) CHANNEL_REC(4, 16);
+  else CHANNEL_REC(8, 8);
+#undef CHANNEL_REC
   return launch_status();
 }

@@ -141,12 +141,52 @@ __global__ void __launch_bounds__(256) act_kernel(const S* __restrict__ in, int6
     out[t * ld_out + i] = from_f32<S>(act1(to_f32(in[t * ld_in + i]), act));
 }
 
+// entry i of x meets entry i / group of g: one gate for every `group` consecutive columns (a head), group 1: one each
 template <class S>
 __global__ void __launch_bounds__(256) gate_kernel(S* __restrict__ x, int64_t ld_x, const S* __restrict__ g, int64_t ld_g,
-                                                   int64_t n, int act) {
+                                                   int64_t n, int act, int64_t group) {
   const int64_t t = blockIdx.y;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
-    x[t * ld_x + i] = from_f32<S>(to_f32(x[t * ld_x + i]) * act1(to_f32(g[t * ld_g + i]), act));
+    x[t * ld_x + i] = from_f32<S>(to_f32(x[t * ld_x + i]) * act1(to_f32(g[t * ld_g + (group > 1 ? i / group : i)]), act));
+}
+
+// out[t, i] = act(in[t, i]) * in[t, inter + i] for any activation of act1
+template <class S>
+__global__ void __launch_bounds__(256) gated_any_kernel(const S* __restrict__ in, S* __restrict__ out, int64_t inter,
+                                                        int64_t ld_in, int act) {
+  const int64_t t = blockIdx.y;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < inter; i += (int64_t)gridDim.x * blockDim.x)
+    out[t * inter + i] = from_f32<S>(act1(to_f32(in[t * ld_in + i]), act) * to_f32(in[t * ld_in + inter + i]));
+}
+
+// Token shift: out[t] = x[t] + (before - x[t]) * mix, `before` the row of the token before in its request: the row
+// above inside a step's portion, the request's kept row (state[slot]) for a portion's first row. The thread that
+// serves a portion's first row then keeps the portion's last row for the next step, so nobody reads the kept row
+// after it has been replaced. A workgroup takes one request and TOK of its rows.
+constexpr int SHIFT_TOK = 8;
+template <class S>
+__global__ void __launch_bounds__(256) token_shift_kernel(const S* __restrict__ x, int64_t ld_x, S* __restrict__ out,
+                                                          int64_t ld_out, S* __restrict__ state,
+                                                          const float* __restrict__ mix, const int32_t* __restrict__ cu,
+                                                          const int32_t* __restrict__ seq_lens,
+                                                          const int32_t* __restrict__ slots, int64_t width) {
+  const int b = blockIdx.y;
+  const int t0 = cu[b], n = cu[b + 1] - t0;
+  const bool starts = seq_lens[b] - n <= 0;   // the request's first token: zeros before it, whatever the slot held
+  const int r0 = blockIdx.x * SHIFT_TOK;
+  if (r0 >= n) return;
+  const int r1 = r0 + SHIFT_TOK < n ? r0 + SHIFT_TOK : n;
+  S* kept = state + (int64_t)slots[b] * width;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+    const float m = mix[i];
+    float before = r0 > 0 ? to_f32(x[(int64_t)(t0 + r0 - 1) * ld_x + i]) : starts ? 0.f : to_f32(kept[i]);
+    for (int r = r0; r < r1; ++r) {
+      const float v = to_f32(x[(int64_t)(t0 + r) * ld_x + i]);
+      out[(int64_t)(t0 + r) * ld_out + i] = from_f32<S>(v + (before - v) * m);
+      before = v;
+    }
+    if (r0 == 0) kept[i] = x[(int64_t)(t0 + n - 1) * ld_x + i];
+  }
 }
 
 }  // namespace
@@ -165,12 +205,22 @@ extern "C" int dinfer_embedding(int dtype, const int32_t* ids, const void* table
   return launch_status();
 }
 
-// act: 0 = silu. Anything else is refused.
+// act: 0 = silu, 2 = gelu in its tanh form (the codes of act1). Anything else is refused.
 extern "C" int dinfer_gated_act(int dtype, int act, const void* in, void* out, int64_t tokens, int64_t inter,
                                 int64_t ld_in, hipStream_t stream) {
   if (tokens <= 0) return OK;
-  if (act != 0) return ERR_UNSUPPORTED;
+  if (act != 0 && act != 2) return ERR_UNSUPPORTED;
   if (inter <= 0 || ld_in < 2 * inter || tokens > 65535 * 1024LL) return ERR_BAD_SHAPE;
+  if (act != 0) {
+    for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
+      const int64_t nt = tokens - t0 < 65535 ? tokens - t0 : 65535;
+      const dim3 grid(blocks_for(inter, 256, 64), (unsigned)nt);
+      DINFER_DISPATCH_DTYPE(dtype, {
+        gated_any_kernel<S><<<grid, 256, 0, stream>>>((const S*)in + t0 * ld_in, (S*)out + t0 * inter, inter, ld_in, act);
+      });
+    }
+    return launch_status();
+  }
   // grid.y is limited to 65535 rows; larger batches are cut into slabs
   for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
     const int64_t nt = tokens - t0 < 65535 ? tokens - t0 : 65535;
@@ -243,16 +293,17 @@ extern "C" int dinfer_embedding_to(int table_dtype, int out_dtype, const int32_t
 }
 
 // x[t, i] *= act(g[t, i]) for i < n: a gate on a block of columns (x and g point at the first column of theirs).
+// group > 1: one gate for every `group` consecutive columns of x (g has n / group columns).
 extern "C" int dinfer_gate(int dtype, int act, void* x, int64_t ld_x, const void* g, int64_t ld_g, int64_t tokens,
-                           int64_t n, hipStream_t stream) {
+                           int64_t n, int64_t group, hipStream_t stream) {
   if (tokens <= 0 || n <= 0) return OK;
   if (act < 0 || act > 4) return ERR_UNSUPPORTED;
-  if (ld_x < n || ld_g < n) return ERR_BAD_SHAPE;
+  if (group < 1 || n % group || ld_x < n || ld_g < n / group) return ERR_BAD_SHAPE;
   for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
     const int64_t nt = tokens - t0 < 65535 ? tokens - t0 : 65535;
     const dim3 grid((unsigned)((n + 1023) / 1024 < 64 ? (n + 1023) / 1024 : 64), (unsigned)nt);
     DINFER_DISPATCH_DTYPE(dtype, {
-      gate_kernel<S><<<grid, 256, 0, stream>>>((S*)x + t0 * ld_x, ld_x, (const S*)g + t0 * ld_g, ld_g, n, act);
+      gate_kernel<S><<<grid, 256, 0, stream>>>((S*)x + t0 * ld_x, ld_x, (const S*)g + t0 * ld_g, ld_g, n, act, group);
     });
   }
   return launch_status();
@@ -272,6 +323,24 @@ extern "C" int dinfer_act(int dtype, int act, const void* in, int64_t ld_in, voi
       act_kernel<S><<<grid, 256, 0, stream>>>((const S*)in + t0 * ld_in, ld_in, (S*)out + t0 * ld_out, ld_out, n, act);
     });
   }
+  return launch_status();
+}
+
+// out[t] = x[t] + (row before - x[t]) * mix for the rows of num_reqs requests (cu_seqlens), the row before a
+// portion's first row taken from state[slots[b]] (zeros for a request that starts), which then takes the portion's
+// last row of x. x, out and state in the step's dtype, mix float [width]; out must not be x. max_rows: the longest
+// portion of the step (or more). seq_lens: the requests' lengths after the step.
+extern "C" int dinfer_token_shift(int dtype, const void* x, int64_t ld_x, void* out, int64_t ld_out, void* state,
+                                  const float* mix, const int32_t* cu_seqlens, const int32_t* seq_lens,
+                                  const int32_t* slots, int num_reqs,
+                                  int64_t max_rows, int64_t width, hipStream_t stream) {
+  if (num_reqs <= 0 || max_rows <= 0) return OK;
+  if (width <= 0 || ld_x < width || ld_out < width || num_reqs > 65535 || x == out) return ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)((max_rows + SHIFT_TOK - 1) / SHIFT_TOK), (unsigned)num_reqs);
+  DINFER_DISPATCH_DTYPE(dtype, {
+    token_shift_kernel<S><<<grid, width >= 256 ? 256 : 64, 0, stream>>>((const S*)x, ld_x, (S*)out, ld_out, (S*)state, mix,
+                                                                        cu_seqlens, seq_lens, slots, width);
+  });
   return launch_status();
 }
 

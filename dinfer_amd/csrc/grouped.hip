@@ -395,16 +395,60 @@ __global__ void __launch_bounds__(256) moe_logits_bf16x8_kernel(const bf16* __re
 
 // A wave per token: the `top` largest of its logits, one after the other (among equals the lowest index), the softmax
 // over the chosen, and the sigmoid of the shared expert's gate logit (z[t, E]) where there is one.
+// all_scores: the scores are the softmax over all E logits; the choice goes by score + correction[e] (correction may
+// be null) and a chosen expert's weight is its score as it is (the weights of a token need not sum to one).
 __global__ void __launch_bounds__(256) moe_topk_kernel(const float* __restrict__ z, int ldz, int tokens, int E, int top,
                                                        int has_shared, int32_t* __restrict__ idx,
-                                                       float* __restrict__ share, float* __restrict__ shared_gate) {
+                                                       float* __restrict__ share, float* __restrict__ shared_gate,
+                                                       int all_scores, const float* __restrict__ correction) {
   __shared__ float zs[4][MAX_EXPERTS];
+  __shared__ float sc[4][MAX_EXPERTS];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * 4 + wave;
   if (t >= tokens) return;   // (no workgroup barrier below)
   float* zw = zs[wave];
   for (int e = lane; e < E; e += 64) zw[e] = z[t * ldz + e];
   if (has_shared && lane == 0) shared_gate[t] = sigmoid(z[t * ldz + E]);
+  if (all_scores) {
+    float* sw = sc[wave];
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zw[e]);   // (a lane reads back what it wrote itself)
+    mx = wave_max(mx);
+    float den = 0.f;
+    for (int e = lane; e < E; e += 64) { const float p = expf(zw[e] - mx); sw[e] = p; den += p; }
+    den = wave_sum(den);
+    for (int e = lane; e < E; e += 64) {
+      const float p = sw[e] / den;
+      sw[e] = p;
+      zw[e] = p + (correction ? correction[e] : 0.f);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    int chosen_e = 0;
+    for (int c = 0; c < top; ++c) {
+      float best = -INFINITY;
+      int be = 0x7fffffff;
+      for (int e = lane; e < E; e += 64) {
+        const float v = zw[e];
+        if (v > best || (v == best && e < be)) { best = v; be = e; }
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oe = __shfl_xor(be, o, 64);
+        if (ov > best || (ov == best && oe < be)) { best = ov; be = oe; }
+      }
+      if (lane == c) chosen_e = be;
+      if (lane == 0 && be < E) zw[be] = -INFINITY;
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (lane < top) {
+      idx[t * top + lane] = chosen_e;
+      share[t * top + lane] = chosen_e < E ? sw[chosen_e] : 0.f;
+    }
+    return;
+  }
   __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
   __builtin_amdgcn_wave_barrier();
   float chosen = 0.f, zmax = 0.f, sum = 0.f;   // lane c keeps the c-th choice
@@ -436,9 +480,11 @@ __global__ void __launch_bounds__(256) moe_topk_kernel(const float* __restrict__
 }
 
 // One workgroup. entries = tokens * top.
+// Experts from `real` on have no weights (their output is their input): their entries are sorted like the others', but
+// no tile is made for them.
 __global__ void __launch_bounds__(1024) moe_scatter_kernel(const int32_t* __restrict__ idx, int entries, int E, int tile_rows,
                                                            int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
-                                                           int32_t* __restrict__ tiles, int max_tiles) {
+                                                           int32_t* __restrict__ tiles, int max_tiles, int real) {
   __shared__ int cnt[MAX_EXPERTS], off[MAX_EXPERTS + 1], tbase[MAX_EXPERTS + 1];
   for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
@@ -449,7 +495,7 @@ __global__ void __launch_bounds__(1024) moe_scatter_kernel(const int32_t* __rest
     for (int e = 0; e < E; ++e) {
       off[e] = o; tbase[e] = tb;
       o += cnt[e];
-      tb += (cnt[e] + tile_rows - 1) / tile_rows;
+      if (e < real) tb += (cnt[e] + tile_rows - 1) / tile_rows;
     }
     off[E] = o; tbase[E] = tb;
   }
@@ -475,12 +521,17 @@ template <class S>
 __global__ void __launch_bounds__(256) moe_combine_kernel(const S* __restrict__ y, int64_t ld_y, const float* __restrict__ share,
                                                           int top, const S* __restrict__ shared, int64_t ld_s,
                                                           const float* __restrict__ shared_gate, S* __restrict__ out,
-                                                          int64_t ld_o, int width) {
+                                                          int64_t ld_o, int width, const int32_t* __restrict__ idx,
+                                                          int real, const S* __restrict__ x, int64_t ld_x) {
   const int64_t t = blockIdx.x;
   const float sg = shared ? (shared_gate ? shared_gate[t] : 1.f) : 0.f;   // no gate: the shared output as it is
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float acc = 0.f;
-    for (int c = 0; c < top; ++c) acc = fmaf(share[t * top + c], to_f32(y[(t * top + c) * ld_y + i]), acc);
+    for (int c = 0; c < top; ++c) {
+      // an expert without weights hands the token's input on
+      const bool same = idx && idx[t * top + c] >= real;
+      acc = fmaf(share[t * top + c], to_f32(same ? x[t * ld_x + i] : y[(t * top + c) * ld_y + i]), acc);
+    }
     if (shared) acc = fmaf(sg, to_f32(shared[t * ld_s + i]), acc);
     out[t * ld_o + i] = from_f32<S>(acc);
   }
@@ -497,7 +548,9 @@ __global__ void __launch_bounds__(256) moe_combine_bf16x8_kernel(const bf16* __r
                                                                  const float* __restrict__ share, int top,
                                                                  const bf16* __restrict__ shared, int64_t ld_s,
                                                                  const float* __restrict__ shared_gate,
-                                                                 bf16* __restrict__ out, int64_t ld_o, int width) {
+                                                                 bf16* __restrict__ out, int64_t ld_o, int width,
+                                                                 const int32_t* __restrict__ idx, int real,
+                                                                 const bf16* __restrict__ x, int64_t ld_x) {
   const int64_t t = blockIdx.x;
   const float sg = shared ? (shared_gate ? shared_gate[t] : 1.f) : 0.f;   // no gate: the shared output as it is
   for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
@@ -505,7 +558,8 @@ __global__ void __launch_bounds__(256) moe_combine_bf16x8_kernel(const bf16* __r
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
     for (int c = 0; c < top; ++c) {
-      const bf16x8 v = *(const bf16x8*)(y + (t * top + c) * ld_y + i);
+      const bool same = idx && idx[t * top + c] >= real;   // an expert without weights hands the token's input on
+      const bf16x8 v = *(const bf16x8*)(same ? x + t * ld_x + i : y + (t * top + c) * ld_y + i);
       const float w = share[t * top + c];
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[j] = fmaf(w, (float)v[j], acc[j]);
@@ -591,7 +645,9 @@ extern "C" int dinfer_moe_tile_rows(int dtype, int64_t entries, int experts, int
 // z: float scratch [tokens, experts + 1].
 extern "C" int dinfer_moe_route(int dtype, const void* x, int64_t ld_x, int64_t tokens, const float* router,
                                 const float* shared_gate_w, int experts, int top, int width, float* z, int32_t* idx,
-                                float* share, float* shared_gate, hipStream_t stream) {
+                                float* share, float* shared_gate, int all_scores, const float* correction,
+                                hipStream_t stream) {
+  // all_scores: softmax over all experts, chosen by score + correction (float [experts] or null), weights the scores
   if (tokens <= 0) return OK;
   if (experts <= 0 || top <= 0 || top > experts || width <= 0 || tokens > 0x7fffffff || !z) return ERR_BAD_SHAPE;
   if (experts > MAX_EXPERTS || top > 64) return ERR_UNSUPPORTED;
@@ -618,36 +674,47 @@ extern "C" int dinfer_moe_route(int dtype, const void* x, int64_t ld_x, int64_t 
   });
   if (launch_status() != OK) return ERR_LAUNCH;
   moe_topk_kernel<<<(unsigned)((tokens + 3) / 4), 256, 0, stream>>>(z, ldz, (int)tokens, experts, top,
-                                                                   shared_gate_w ? 1 : 0, idx, share, shared_gate);
+                                                                   shared_gate_w ? 1 : 0, idx, share, shared_gate,
+                                                                   all_scores, correction);
   return launch_status();
 }
 
 extern "C" int dinfer_moe_scatter(const int32_t* idx, int64_t entries, int experts, int tile_rows, int32_t* offsets,
-                                  int32_t* perm, int32_t* tiles, int64_t max_tiles, hipStream_t stream) {
+                                  int32_t* perm, int32_t* tiles, int64_t max_tiles, int real_experts,
+                                  hipStream_t stream) {
+  // real_experts < experts: the experts from there on get no tiles (0 or less: all are real)
+  if (real_experts <= 0 || real_experts > experts) real_experts = experts;
   if (entries <= 0) return OK;
   if (experts <= 0 || tile_rows <= 0 || entries > 0x7fffffff ||
       max_tiles < (entries + tile_rows - 1) / tile_rows + experts)
     return ERR_BAD_SHAPE;
   if (experts > MAX_EXPERTS) return ERR_UNSUPPORTED;
-  moe_scatter_kernel<<<1, 1024, 0, stream>>>(idx, (int)entries, experts, tile_rows, offsets, perm, tiles, (int)max_tiles);
+  moe_scatter_kernel<<<1, 1024, 0, stream>>>(idx, (int)entries, experts, tile_rows, offsets, perm, tiles, (int)max_tiles,
+                                             real_experts);
   return launch_status();
 }
 
 extern "C" int dinfer_moe_combine(int dtype, const void* y, int64_t ld_y, const float* share, int top, const void* shared,
                                   int64_t ld_s, const float* shared_gate, void* out, int64_t ld_o, int64_t tokens,
-                                  int width, hipStream_t stream) {
+                                  int width, const int32_t* idx, int real_experts, const void* x, int64_t ld_x,
+                                  hipStream_t stream) {
+  // idx (may be null) [tokens, top] with real_experts: a choice from real_experts on adds its share of x[t], the
+  // token's input, instead of a row of y.
   if (tokens <= 0) return OK;
-  if (top <= 0 || width <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
+  if (top <= 0 || width <= 0 || tokens > 0x7fffffff || (idx && (!x || ld_x < width))) return ERR_BAD_SHAPE;
   const bool vec = dtype == DT_BF16 && width % 8 == 0 && ld_y % 8 == 0 && ld_o % 8 == 0 && (!shared || ld_s % 8 == 0) &&
-                   ((uintptr_t)y % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)shared % 16) == 0;
+                   ((uintptr_t)y % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)shared % 16) == 0 &&
+                   (!idx || (ld_x % 8 == 0 && ((uintptr_t)x % 16) == 0));
   if (vec) {
     moe_combine_bf16x8_kernel<<<(unsigned)tokens, width >= 2048 ? 256 : 64, 0, stream>>>(
-        (const bf16*)y, ld_y, share, top, (const bf16*)shared, ld_s, shared_gate, (bf16*)out, ld_o, width);
+        (const bf16*)y, ld_y, share, top, (const bf16*)shared, ld_s, shared_gate, (bf16*)out, ld_o, width, idx,
+        real_experts, (const bf16*)x, ld_x);
     return launch_status();
   }
   DINFER_DISPATCH_DTYPE(dtype, {
     moe_combine_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)y, ld_y, share, top, (const S*)shared, ld_s,
-                                                               shared_gate, (S*)out, ld_o, width);
+                                                               shared_gate, (S*)out, ld_o, width, idx, real_experts,
+                                                               (const S*)x, ld_x);
   });
   return launch_status();
 }

@@ -40,10 +40,12 @@ __global__ void __launch_bounds__(256) latent_post_kernel(
     const S* __restrict__ proj, int64_t ld, int q_off, int c_off, int H, int dn, int dr, int R,
     const void* __restrict__ gain, int wf32, float eps, const int32_t* __restrict__ positions,
     const float* __restrict__ cos_sin, int rot, S* __restrict__ qa, int64_t ld_qa, S* __restrict__ cache,
-    S* __restrict__ cache_t, int page, const int64_t* __restrict__ slots) {
+    S* __restrict__ cache_t, int page, const int64_t* __restrict__ slots, int style, const S* __restrict__ qsrc,
+    int64_t ld_qs) {
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
   const S* row = proj + t * ld;
+  const S* qrow = qsrc ? qsrc + t * ld_qs : row;   // the queries may come from a product of their own
   const int pos = positions[t];
   const float* cs = cos_sin ? cos_sin + (int64_t)pos * rot : nullptr;
   const int half = rot / 2;
@@ -51,20 +53,24 @@ __global__ void __launch_bounds__(256) latent_post_kernel(
   const int pairs = dr / 2;
   for (int i = threadIdx.x; i < H * pairs; i += blockDim.x) {
     const int h = i / pairs, j = i - h * pairs;
-    const S* src = row + q_off + (int64_t)h * (dn + dr) + dn + 2 * j;
-    float u = to_f32(src[0]), v = to_f32(src[1]);
+    // style 1: entries (2j, 2j+1) pair up; style 0: entry j pairs with j + rot/2 (the entries from rot on, which do
+    // not turn, are walked two by two in either style)
+    const bool halves = style == 0 && j < half;
+    const int ia = halves ? j : 2 * j, ib = halves ? j + half : 2 * j + 1;
+    const S* src = qrow + q_off + (int64_t)h * (dn + dr) + dn;
+    float u = to_f32(src[ia]), v = to_f32(src[ib]);
     if (cs && j < half) {
       const float c = cs[j], s = cs[half + j];
       const float a = rotated_first(u, v, c, s), b = rotated_second(u, v, c, s);
       u = a; v = b;
     }
-    S* dst = qa + t * ld_qa + (int64_t)h * (R + dr) + R + 2 * j;
-    dst[0] = from_f32<S>(u);
-    dst[1] = from_f32<S>(v);
+    S* dst = qa + t * ld_qa + (int64_t)h * (R + dr) + R;
+    dst[ia] = from_f32<S>(u);
+    dst[ib] = from_f32<S>(v);
   }
   if (dr & 1) {   // an odd last entry passes unchanged
     for (int h = threadIdx.x; h < H; h += blockDim.x)
-      qa[t * ld_qa + (int64_t)h * (R + dr) + R + dr - 1] = row[q_off + (int64_t)h * (dn + dr) + dn + dr - 1];
+      qa[t * ld_qa + (int64_t)h * (R + dr) + R + dr - 1] = qrow[q_off + (int64_t)h * (dn + dr) + dn + dr - 1];
   }
   if (c_off < 0 || !slots) return;
   const int64_t slot = slots[t];
@@ -82,14 +88,16 @@ __global__ void __launch_bounds__(256) latent_post_kernel(
     if (dst_t) dst_t[(int64_t)i * page] = v;
   }
   for (int j = threadIdx.x; j < pairs; j += blockDim.x) {
-    float u = to_f32(c[R + 2 * j]), v = to_f32(c[R + 2 * j + 1]);
+    const bool halves = style == 0 && j < half;
+    const int ia = halves ? j : 2 * j, ib = halves ? j + half : 2 * j + 1;
+    float u = to_f32(c[R + ia]), v = to_f32(c[R + ib]);
     if (cs && j < half) {
       const float co = cs[j], si = cs[half + j];
       const float a = rotated_first(u, v, co, si), b = rotated_second(u, v, co, si);
       u = a; v = b;
     }
-    dst[R + 2 * j] = from_f32<S>(u);
-    dst[R + 2 * j + 1] = from_f32<S>(v);
+    dst[R + ia] = from_f32<S>(u);
+    dst[R + ib] = from_f32<S>(v);
   }
   if ((dr & 1) && threadIdx.x == 0) dst[R + dr - 1] = c[R + dr - 1];
 }
@@ -676,18 +684,23 @@ __global__ void __launch_bounds__(128) latent_attn_merge_kernel(const float* __r
 // at c_off (R latent, then dr shared key part; c_off < 0: this layer has none and nothing is written to the cache).
 // cos_sin [positions, rot] = [cos | sin] of rot/2 angles (null: no rotation); the first `rot` entries of a rotated part
 // turn. qa [T, ld_qa]: head h at h*(R+dr); its last dr entries are written here. cache [blocks*page, R+dr].
+// style: 1 pairs (2i, 2i+1), 0 pairs (i, i + rot/2). q_src (may be null: the queries are in proj): [T, ld_qs], the
+// queries at column q_off of it.
 extern "C" int dinfer_latent_post(int dtype, const void* proj, int64_t tokens, int64_t ld, int q_off, int c_off, int heads,
                                   int dn, int dr, int R, const void* gain, int w_f32, float eps,
                                   const int32_t* positions, const float* cos_sin, int rot, void* qa, int64_t ld_qa,
-                                  void* cache, void* cache_t, int page_size, const int64_t* slots, hipStream_t stream) {
+                                  void* cache, void* cache_t, int page_size, const int64_t* slots, int style,
+                                  const void* q_src, int64_t ld_qs, hipStream_t stream) {
   if (tokens <= 0) return OK;
+  if (style != 0 && style != 1) return ERR_UNSUPPORTED;
   if (heads <= 0 || dn < 0 || dr < 0 || R <= 0 || rot < 0 || rot > dr || (rot & 1) || tokens > 0x7fffffff ||
       ld_qa < (int64_t)heads * (R + dr) || (cache_t && page_size <= 0))
     return ERR_BAD_SHAPE;
   DINFER_DISPATCH_DTYPE(dtype, {
     latent_post_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>((const S*)proj, ld, q_off, c_off, heads, dn, dr, R, gain,
                                                                w_f32, eps, positions, cos_sin, rot, (S*)qa, ld_qa,
-                                                               (S*)cache, (S*)cache_t, page_size, slots);
+                                                               (S*)cache, (S*)cache_t, page_size, slots, style,
+                                                               (const S*)q_src, ld_qs);
   });
   return launch_status();
 }

@@ -45,7 +45,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
     const void* __restrict__ wk, int wf32, float eps, float w_offset, const int32_t* __restrict__ pos,
     const float* __restrict__ cos_sin, int rot, int style, S* __restrict__ k_cache, S* __restrict__ v_cache,
     const int64_t* __restrict__ slots, int H, int Hkv, int D, int page, int Dv, const float* __restrict__ bias,
-    float temp_coef, int temp_every) {
+    float temp_coef, int temp_every, const float* __restrict__ head_scale) {
   __shared__ float xs[WAVES][MAX_D];
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -90,6 +90,8 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
       float inv = 1.f / sqrtf(ss / (float)D + eps);
       // a query grows with its position: 1 + coef ln(floor((p + 1) / every) + 1)
       if (is_q && temp_every > 0) inv *= 1.f + temp_coef * logf((float)((pos[t] + 1) / temp_every) + 1.f);
+      // a temperature a query head: the head's scores are multiplied by it, so its query is
+      if (is_q && head_scale) inv *= head_scale[item];
       // each lane rescales only the entries it wrote itself
       for (int d = lane; d < D; d += 64) x[d] = x[d] * inv * (ld_param<S>(w, d, wf32) + w_offset);
     }
@@ -299,7 +301,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
     const void* __restrict__ wk, int wf32, float eps, float w_offset, const int32_t* __restrict__ pos,
     const float* __restrict__ cos_sin, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
     const int64_t* __restrict__ slots, int H, int Hkv, int page, int tokens, int gather_v,
-    const float* __restrict__ bias, float temp_coef, int temp_every) {
+    const float* __restrict__ bias, float temp_coef, int temp_every, const float* __restrict__ head_scale) {
   constexpr int D = LPH * 8, HALF = D / 2, HPW = 64 / LPH;  // heads per wave
   if ((int)blockIdx.x >= tokens) {
     const int j = (int)blockIdx.x - tokens;
@@ -407,6 +409,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
     float inv = (qk && w) ? 1.f / sqrtf(ss / (float)D + eps) : 1.f;
     // a query grows with its position: 1 + coef ln(floor((p + 1) / every) + 1)
     if (is_q && w && temp_every > 0) inv *= 1.f + temp_coef * logf((float)((pos[t] + 1) / temp_every) + 1.f);
+    if (is_q && w && head_scale) inv *= head_scale[item];
     float y[8], other[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) y[e] = (qk && w) ? x[e] * inv * g[e] : x[e];
@@ -433,7 +436,9 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
                                float w_offset, const int32_t* positions, const float* cos_sin, int rotary_dim,
                                int style, void* k_cache, void* v_cache, const int64_t* slot_mapping, int heads,
                                int kv_heads, int head_dim, int page_size, int token_runs, int v_dim,
-                               const float* bias, float temp_coef, int temp_every, hipStream_t stream) {
+                               const float* bias, float temp_coef, int temp_every, const float* head_scale,
+                               hipStream_t stream) {
+  // head_scale (may be null): float [heads], q of head h is multiplied by head_scale[h] with the norm (gains needed).
   // bias (may be null): float [q heads | k heads | v heads], added to the product's output before anything else.
   // temp_every > 0: q is multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1) with the norm (gains needed).
   // v_dim: the size of a value head, 0 for head_dim. v_cache may be null beside a k_cache (values are not stored).
@@ -448,10 +453,10 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   if ((q_gain == nullptr) != (k_gain == nullptr)) return ERR_BAD_SHAPE;
   const int items = heads + 2 * kv_heads;
   const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES - 1) / WAVES));
-  if (temp_every > 0 && !q_gain) return ERR_UNSUPPORTED;
+  if ((temp_every > 0 || head_scale) && !q_gain) return ERR_UNSUPPORTED;
   const bool whole_head_neox = style == 0 && head_dim % 8 == 0 && (!cos_sin || rotary_dim == head_dim) &&
                                v_dim == head_dim && (v_cache || !slot_mapping);
-  const bool plain_head = !bias && temp_every <= 0;   // what the kernels of 2-byte accesses for whole heads take
+  const bool plain_head = !bias && temp_every <= 0 && !head_scale;   // what the kernels of 2-byte accesses for whole heads take
   const bool vec_ok = dtype == DT_BF16 && (head_dim == 64 || head_dim == 128 || head_dim == 256) && ld % 8 == 0 &&
                       q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
                       ((uintptr_t)q_gain % 16) == 0 && ((uintptr_t)k_gain % 16) == 0 && ((uintptr_t)cos_sin % 16) == 0 &&
@@ -469,7 +474,7 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   qkv_post_vec_kernel<LPH_><<<vgrid, WAVES * 64, 0, stream>>>(                                                         \
       (bf16*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps, w_offset, positions, cos_sin, (bf16*)k_cache, \
       (bf16*)v_cache, slot_mapping, heads, kv_heads, page_size, (int)tokens, (int)gather_v, bias, temp_coef,       \
-      temp_every)
+      temp_every, head_scale)
     if (lph == 8) DINFER_QKV_VEC(8);
     else if (lph == 16) DINFER_QKV_VEC(16);
     else DINFER_QKV_VEC(32);
@@ -498,7 +503,8 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
     qkv_post_kernel<S><<<grid, WAVES * 64, 0, stream>>>((S*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps,
                                                         w_offset, positions, cos_sin, rotary_dim, style, (S*)k_cache,
                                                         (S*)v_cache, slot_mapping, heads, kv_heads, head_dim,
-                                                        page_size, v_dim, bias, temp_coef, temp_every);
+                                                        page_size, v_dim, bias, temp_coef, temp_every,
+                                                        head_scale);
   });
   return launch_status();
 }

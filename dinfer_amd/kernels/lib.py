@@ -27,21 +27,22 @@ SIGNATURES = {
     "dinfer_embedding_to": ("elementwise", [_I, _I, _P, _P, _P, _L, _L, _L, _F, _P, _P, _P]),
     "dinfer_act": ("elementwise", [_I, _I, _P, _L, _P, _L, _L, _L, _P]),
     "dinfer_layernorm": ("norm", [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _L, _L, _L, _L, _F, _P]),
-    "dinfer_latent_post": ("latent", [_I, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P, _I, _F, _P, _P, _I, _P, _L, _P, _P, _I, _P, _P]),
+    "dinfer_latent_post": ("latent", [_I, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P, _I, _F, _P, _P, _I, _P, _L, _P, _P, _I, _P, _I,
+                                      _P, _L, _P]),
     "dinfer_latent_mfma_supports": ("latent", [_I, _I, _I]),
     "dinfer_latent_attn_mfma": ("latent", [_P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _I, _P]),
     "dinfer_latent_attn_ref": ("latent", [_I, _P, _L, _P, _L, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _P]),
     "dinfer_heads_nt": ("grouped", [_I, _P, _L, _L, _P, _L, _L, _P, _L, _L, _L, _L, _L, _L, _P, _L, _P]),
     "dinfer_experts_nt": ("grouped", [_I, _I, _P, _L, _P, _L, _L, _P, _L, _L, _L, _P, _L, _I, _P, _P, _I, _I, _P]),
     "dinfer_moe_tile_rows": ("grouped", [_I, _L, _I, _L, _L]),
-    "dinfer_moe_route": ("grouped", [_I, _P, _L, _L, _P, _P, _I, _I, _I, _P, _P, _P, _P, _P]),
-    "dinfer_moe_scatter": ("grouped", [_P, _L, _I, _I, _P, _P, _P, _L, _P]),
-    "dinfer_moe_combine": ("grouped", [_I, _P, _L, _P, _I, _P, _L, _P, _P, _L, _L, _I, _P]),
+    "dinfer_moe_route": ("grouped", [_I, _P, _L, _L, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P]),
+    "dinfer_moe_scatter": ("grouped", [_P, _L, _I, _I, _P, _P, _P, _L, _I, _P]),
+    "dinfer_moe_combine": ("grouped", [_I, _P, _L, _P, _I, _P, _L, _P, _P, _L, _L, _I, _P, _I, _P, _L, _P]),
     "dinfer_rmsnorm": ("norm", [_I, _P, _P, _P, _P, _I, _P, _L, _L, _L, _L, _F, _F, _P]),
     "dinfer_qkv_post": (
         "rope",
         [_I, _P, _L, _L, _L, _L, _L, _P, _P, _I, _F, _F, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I,
-         _P],
+         _P, _P],
     ),
     "dinfer_attn_paged_ref": (
         "attention_ref",
@@ -51,6 +52,10 @@ SIGNATURES = {
         "attention_ref",
         [_I, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _P, _F, _I, _I, _I, _I, _I, _F, _P],
     ),
+    "dinfer_attn_paged_diff": (
+        "attention_ref",
+        [_I, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P],
+    ),
     "dinfer_rmsnorm_stream": ("norm", [_P, _I, _L, _P, _F, _F, _F, _P, _I, _L, _P, _P, _I, _P, _I, _F, _F, _L, _L, _P]),
     "dinfer_axpby": ("elementwise", [_I, _P, _L, _F, _P, _L, _F, _P, _L, _L, _L, _P]),
     "dinfer_add_rows": ("elementwise", [_P, _I, _L, _P, _I, _L, _P, _I, _L, _L, _P]),
@@ -58,8 +63,11 @@ SIGNATURES = {
                                     _I, _I, _F, _F, _P]),
     "dinfer_delta_conv_update": ("delta", [_I, _P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _P]),
     "dinfer_delta_recurrence": ("delta", [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P]),
-    "dinfer_delta_out": ("delta", [_I, _P, _L, _P, _L, _L, _P, _P, _L, _L, _L, _I, _I, _F, _F, _P]),
-    "dinfer_gate": ("elementwise", [_I, _I, _P, _L, _P, _L, _L, _L, _P]),
+    "dinfer_delta_out": ("delta", [_I, _P, _L, _P, _L, _L, _P, _P, _L, _L, _L, _I, _I, _F, _F, _I, _I, _P]),
+    "dinfer_channel_delta_prep": ("delta", [_I, _P, _L, _L, _L, _L, _L, _L, _P, _P, _P, _I, _P, _L, _L, _I, _I, _F, _F, _P]),
+    "dinfer_channel_delta_recurrence": ("delta", [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P]),
+    "dinfer_gate": ("elementwise", [_I, _I, _P, _L, _P, _L, _L, _L, _L, _P]),
+    "dinfer_token_shift": ("elementwise", [_I, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _L, _L, _P]),
     "dinfer_rot_widen": ("decay", [_I, _P, _L, _L, _L, _L, _P, _P, _I, _F, _P, _L, _L, _I, _I, _I, _P]),
     "dinfer_conv_silu": ("decay", [_I, _P, _L, _L, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _L, _I, _I, _I, _P]),
     "dinfer_decay_recurrence": ("decay", [_P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I,

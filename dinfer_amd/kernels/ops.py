@@ -81,7 +81,7 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, src: to
     return out
 
 
-GATED_ACTS = {"silu": 0}   # activations the gated kernels know -> their code in the C interface
+GATED_ACTS = {"silu": 0, "gelu_tanh": 2}   # activations the gated kernels know -> their code in the C interface
 MAX_HEAD_DIM = 512         # the largest head the norm / rotation / plain attention kernels hold in registers
 
 
@@ -170,16 +170,34 @@ def act(x: torch.Tensor, out: torch.Tensor, tokens: int, kind: str) -> torch.Ten
     return out
 
 
-def gate(x: torch.Tensor, g: torch.Tensor, tokens: int, kind: str) -> torch.Tensor:
-    """x[t, i] *= act(g[t, i]) in place; x and g are views of equally many columns (blocks of wider buffers)."""
+def gate(x: torch.Tensor, g: torch.Tensor, tokens: int, kind: str, group: int = 1) -> torch.Tensor:
+    """x[t, i] *= act(g[t, i // group]) in place; x and g are views (blocks of wider buffers), g of a `group`-th of
+    x's columns: one gate for every `group` consecutive columns (a head), or one each."""
     _need_gpu(x, g)
     if kind not in ACTS:
         raise lib.KernelError(f"activation {kind!r} has no kernel (known: {sorted(ACTS)})")
     n = x.shape[1]
-    assert g.shape[1] == n and x.dtype == g.dtype and x.shape[0] >= tokens and g.shape[0] >= tokens
+    assert group >= 1 and g.shape[1] * group == n and x.dtype == g.dtype and x.shape[0] >= tokens and g.shape[0] >= tokens
     lib.call("dinfer_gate", dtype_code(x.dtype), ACTS[kind], x.data_ptr(), _rows(x), g.data_ptr(), _rows(g), tokens, n,
-             _stream())
+             group, _stream())
     return x
+
+
+def token_shift(x: torch.Tensor, out: torch.Tensor, state: torch.Tensor, mix: torch.Tensor, *, cu_seqlens: torch.Tensor,
+                seq_lens: torch.Tensor, state_slots: torch.Tensor, num_reqs: int, max_rows: int) -> torch.Tensor:
+    """out[t] = x[t] + (x of the token before - x[t]) * mix, per request: inside a portion the row above, for its first
+    row the request's kept row state[slot] (zeros where the request starts), which then takes the portion's last row.
+    state [slots, width] in x's dtype, mix float32 [width]; max_rows: the longest portion of the step."""
+    _need_gpu(x, out, state, mix, cu_seqlens, seq_lens, state_slots)
+    width = mix.numel()
+    assert mix.dtype == torch.float32 and mix.is_contiguous()
+    assert x.dtype == out.dtype == state.dtype and state.is_contiguous() and state.shape[1] == width
+    assert x.shape[1] >= width and out.shape[1] >= width and x.data_ptr() != out.data_ptr()
+    assert cu_seqlens.dtype == seq_lens.dtype == state_slots.dtype == torch.int32
+    lib.call("dinfer_token_shift", dtype_code(x.dtype), x.data_ptr(), _rows(x), out.data_ptr(), _rows(out),
+             state.data_ptr(), mix.data_ptr(), cu_seqlens.data_ptr(), seq_lens.data_ptr(), state_slots.data_ptr(),
+             num_reqs, max_rows, width, _stream())
+    return out
 
 
 def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, eps: float,
@@ -328,15 +346,58 @@ def delta_recurrence(work: torch.Tensor, state: torch.Tensor, out: torch.Tensor,
 
 
 def delta_out(o: torch.Tensor, proj: torch.Tensor, g_off: int, weight: torch.Tensor, out: torch.Tensor, tokens: int, *,
-              heads: int, vdim: int, eps: float, col_off: int = 0, out_scale: float = 1.0) -> torch.Tensor:
-    """out[t, col_off + h vdim + d] = o / rms_d(o) * weight[d] * silu(proj[t, g_off + h vdim + d]) * out_scale."""
+              heads: int, vdim: int, eps: float, col_off: int = 0, out_scale: float = 1.0, gate: str = "silu") -> torch.Tensor:
+    """out[t, col_off + h vdim + d] = o / rms_d(o) * weight[d] * silu(proj[t, g_off + h vdim + d]) * out_scale.
+    weight of heads * vdim entries: a head's own gains at h vdim. gate: "silu" or "sigmoid"."""
     _need_gpu(o, proj, weight, out)
-    assert o.dtype == torch.float32 and weight.dtype == torch.float32 and weight.numel() == vdim
+    per_head = weight.numel() == heads * vdim and heads > 1
+    assert gate in ("silu", "sigmoid")
+    assert o.dtype == torch.float32 and weight.dtype == torch.float32 and (per_head or weight.numel() == vdim)
     assert proj.dtype == out.dtype and min(o.shape[0], proj.shape[0], out.shape[0]) >= tokens
     assert g_off + heads * vdim <= proj.shape[1] and col_off + heads * vdim <= out.shape[1]
     lib.call("dinfer_delta_out", dtype_code(out.dtype), o.data_ptr(), _rows(o), proj.data_ptr(), _rows(proj), g_off,
              weight.data_ptr(), out.data_ptr(), _rows(out), col_off, tokens, heads, vdim, float(eps), float(out_scale),
-             _stream())
+             int(per_head), 1 if gate == "sigmoid" else 0, _stream())
+    return out
+
+
+# ---- delta rule with a decay and a removal rate a key channel ----------------------------------------
+CHANNEL_DELTA_MAX_LOW = 512     # the largest inner size of the decay's low-rank projection
+
+
+def channel_delta_work_columns(heads: int, dim: int) -> int:
+    """Columns of the float rows between the two kernels: r * w | u | k | w | a * u | v | c1 | c2."""
+    return 6 * heads * dim + 2 * heads
+
+
+def channel_delta_prep(proj: torch.Tensor, tokens: int, *, r_off: int, k_off: int, v_off: int, a_off: int, low_off: int,
+                       a_bias: torch.Tensor, w2: torch.Tensor, w0: torch.Tensor, work: torch.Tensor, heads: int, dim: int,
+                       eps: float, rate: float) -> None:
+    """From the step's projections: the unit key u = k / sqrt(sum k^2 + eps), the removal rate a = sigmoid(. + a_bias),
+    the decay w = exp(-rate * sigmoid(w2 tanh(low) + w0)), and what the recurrence reads of them, in float32."""
+    _need_gpu(proj, a_bias, w2, w0, work)
+    hd = heads * dim
+    low = w2.shape[1]
+    assert a_bias.dtype == w2.dtype == w0.dtype == torch.float32 and w2.is_contiguous()
+    assert a_bias.numel() == hd == w0.numel() and w2.shape[0] == hd
+    assert work.dtype == torch.float32 and work.shape[0] >= tokens and work.shape[1] >= channel_delta_work_columns(heads, dim)
+    assert proj.shape[0] >= tokens and max(r_off, k_off, v_off, a_off) + hd <= proj.shape[1] and low_off + low <= proj.shape[1]
+    lib.call("dinfer_channel_delta_prep", dtype_code(proj.dtype), proj.data_ptr(), _rows(proj), r_off, k_off, v_off, a_off,
+             low_off, a_bias.data_ptr(), w2.data_ptr(), w0.data_ptr(), low, work.data_ptr(), _rows(work), tokens, heads,
+             dim, float(eps), float(rate), _stream())
+
+
+def channel_delta_recurrence(work: torch.Tensor, state: torch.Tensor, out: torch.Tensor, *, state_slots: torch.Tensor,
+                             cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, num_reqs: int, heads: int,
+                             dim: int) -> torch.Tensor:
+    """S <- diag(w) S - (a u)(u^T S) + k v^T, o = S^T r over each request's rows of the step. state [slots, heads, dim,
+    dim] float32 (a head's matrix transposed), updated in place; out [T, heads * dim] float32."""
+    _need_gpu(work, state, out, state_slots, cu_seqlens, seq_lens)
+    assert work.dtype == state.dtype == out.dtype == torch.float32 and state.is_contiguous()
+    assert tuple(state.shape[1:]) == (heads, dim, dim) and out.shape[1] >= heads * dim
+    assert work.shape[1] >= channel_delta_work_columns(heads, dim)
+    lib.call("dinfer_channel_delta_recurrence", work.data_ptr(), _rows(work), state.data_ptr(), state_slots.data_ptr(),
+             cu_seqlens.data_ptr(), seq_lens.data_ptr(), out.data_ptr(), _rows(out), num_reqs, heads, dim, _stream())
     return out
 
 
@@ -492,14 +553,18 @@ def latent_cache_shape(blocks: int, page_size: int, rank: int, rot_dim: int) -> 
 def latent_post(proj: torch.Tensor, tokens: int, *, heads: int, dim: int, rot_dim: int, rank: int, q_off: int,
                 c_off: int | None, gain: torch.Tensor | None, eps: float, positions: torch.Tensor,
                 cos_sin: torch.Tensor | None, rotary_dim: int, qa: torch.Tensor, cache: torch.Tensor | None,
-                slot_mapping: torch.Tensor | None, cache_t: torch.Tensor | None = None) -> None:
+                slot_mapping: torch.Tensor | None, cache_t: torch.Tensor | None = None, style: int = 1,
+                q_src: torch.Tensor | None = None) -> None:
     """From the step's projections: every head's rotated query part goes, rotated, into qa (head h at h*(rank+rot_dim),
     behind the rank entries the caller fills), and, where the layer has a down projection of its own (c_off), the
     token's latent (RMS-normed with `gain`) and rotated shared key part go to its cache slot (the latent also into
-    cache_t [blocks, rank, page], the pages transposed, where that is given)."""
-    _need_gpu(proj, gain, positions, cos_sin, qa, cache, slot_mapping, cache_t)
+    cache_t [blocks, rank, page], the pages transposed, where that is given). style: 1 turns pairs (2i, 2i+1), 0 pairs
+    (i, i + rotary_dim/2). q_src: the queries come from this buffer (at its column q_off) instead of from proj."""
+    _need_gpu(proj, gain, positions, cos_sin, qa, cache, slot_mapping, cache_t, q_src)
     assert proj.shape[0] >= tokens and qa.shape[0] >= tokens and qa.dtype == proj.dtype
-    assert q_off + heads * (dim + rot_dim) <= proj.shape[1] and qa.shape[1] >= heads * (rank + rot_dim)
+    qs = proj if q_src is None else q_src
+    assert qs.dtype == proj.dtype and qs.shape[0] >= tokens
+    assert q_off + heads * (dim + rot_dim) <= qs.shape[1] and qa.shape[1] >= heads * (rank + rot_dim)
     assert positions.dtype == torch.int32 and positions.numel() >= tokens
     if cos_sin is not None:
         assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rotary_dim
@@ -516,7 +581,8 @@ def latent_post(proj: torch.Tensor, tokens: int, *, heads: int, dim: int, rot_di
              c_off if write else -1, heads, dim, rot_dim, rank, _ptr(gain) if write else 0,
              _is_param_f32(gain, proj.dtype) if write else 0, float(eps), positions.data_ptr(), _ptr(cos_sin),
              rotary_dim if cos_sin is not None else 0, qa.data_ptr(), _rows(qa), _ptr(cache) if write else 0,
-             _ptr(cache_t) if write else 0, cache.shape[1] if write else 0, _ptr(slot_mapping) if write else 0, _stream())
+             _ptr(cache_t) if write else 0, cache.shape[1] if write else 0, _ptr(slot_mapping) if write else 0,
+             int(style), _ptr(q_src), _rows(q_src) if q_src is not None else 0, _stream())
 
 
 def _check_latent(qa, out, cache, block_table, cu_seqlens, seq_lens, num_reqs, tokens, heads, rank, rot_dim, page_size):
@@ -605,11 +671,16 @@ def moe_max_tiles(entries: int, experts: int, tile_rows: int) -> int:
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, shared_gate_w: torch.Tensor | None, idx: torch.Tensor,
-              share: torch.Tensor, shared_gate: torch.Tensor | None, tokens: int, top: int, z: torch.Tensor) -> None:
+              share: torch.Tensor, shared_gate: torch.Tensor | None, tokens: int, top: int, z: torch.Tensor,
+              all_scores: bool = False, correction: torch.Tensor | None = None) -> None:
     """Per token: logits x @ router.T in float (router float32 [experts, width]), idx[t] the `top` largest (lowest index
     among equals), share[t] the softmax over them; shared_gate[t] = sigmoid(x . shared_gate_w) where that is given.
-    z: float32 scratch of tokens * (experts + 1) for the logits."""
-    _need_gpu(x, router, shared_gate_w, idx, share, shared_gate, z)
+    z: float32 scratch of tokens * (experts + 1) for the logits. all_scores: the scores are the softmax over all
+    experts, the choice goes by score + correction (float32 [experts], or none) and share[t] holds the chosen scores
+    as they are."""
+    _need_gpu(x, router, shared_gate_w, idx, share, shared_gate, z, correction)
+    if correction is not None:
+        assert all_scores and correction.dtype == torch.float32 and correction.numel() == router.shape[0]
     experts, width = router.shape
     assert router.dtype == torch.float32 and router.is_contiguous() and x.shape[1] == width and x.shape[0] >= tokens
     assert idx.dtype == torch.int32 and share.dtype == torch.float32 and idx.is_contiguous() and share.is_contiguous()
@@ -620,13 +691,14 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, shared_gate_w: torch.Tensor
         assert shared_gate is None or (shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens)
     lib.call("dinfer_moe_route", dtype_code(x.dtype), x.data_ptr(), _rows(x), tokens, router.data_ptr(),
              _ptr(shared_gate_w), experts, top, width, z.data_ptr(), idx.data_ptr(), share.data_ptr(),
-             _ptr(shared_gate) if shared_gate_w is not None else 0, _stream())
+             _ptr(shared_gate) if shared_gate_w is not None else 0, int(all_scores), _ptr(correction), _stream())
 
 
 def moe_scatter(idx: torch.Tensor, entries: int, experts: int, offsets: torch.Tensor, perm: torch.Tensor,
-                tiles: torch.Tensor, tile_rows: int) -> None:
+                tiles: torch.Tensor, tile_rows: int, real_experts: int | None = None) -> None:
     """Sorts the entries (token * top + choice) by expert: offsets [experts + 1], perm [entries] (sorted place -> entry),
-    tiles [n, 2] the work list of experts_nt ((expert, first sorted place) per row tile, -1 beyond the last)."""
+    tiles [n, 2] the work list of experts_nt ((expert, first sorted place) per row tile, -1 beyond the last).
+    real_experts: the experts from there on have no weights and get no tiles."""
     _need_gpu(idx, offsets, perm, tiles)
     assert idx.dtype == offsets.dtype == perm.dtype == tiles.dtype == torch.int32
     assert idx.numel() >= entries and perm.numel() >= entries and offsets.numel() >= experts + 1
@@ -634,7 +706,7 @@ def moe_scatter(idx: torch.Tensor, entries: int, experts: int, offsets: torch.Te
     n = moe_max_tiles(entries, experts, tile_rows)
     assert tiles.shape[0] >= n
     lib.call("dinfer_moe_scatter", idx.data_ptr(), entries, experts, tile_rows, offsets.data_ptr(), perm.data_ptr(),
-             tiles.data_ptr(), n, _stream())
+             tiles.data_ptr(), n, int(real_experts or experts), _stream())
 
 
 def experts_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, entries: int, tiles: torch.Tensor,
@@ -658,9 +730,15 @@ def experts_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, entries: int
 
 
 def moe_combine(y: torch.Tensor, share: torch.Tensor, top: int, shared: torch.Tensor | None,
-                shared_gate: torch.Tensor | None, out: torch.Tensor, tokens: int) -> torch.Tensor:
-    """out[t] = sum_c share[t, c] * y[t * top + c] (+ shared_gate[t] * shared[t], or + shared[t] without a gate)."""
-    _need_gpu(y, share, shared, shared_gate, out)
+                shared_gate: torch.Tensor | None, out: torch.Tensor, tokens: int, idx: torch.Tensor | None = None,
+                real_experts: int = 0, x: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = sum_c share[t, c] * y[t * top + c] (+ shared_gate[t] * shared[t], or + shared[t] without a gate).
+    idx, real_experts, x: a choice idx[t, c] >= real_experts stands for an expert whose output is its input: x[t] takes
+    the place of y[t * top + c]."""
+    _need_gpu(y, share, shared, shared_gate, out, idx, x)
+    if idx is not None:
+        assert idx.dtype == torch.int32 and idx.numel() >= tokens * top and x is not None
+        assert x.dtype == out.dtype and x.shape[1] >= out.shape[1] and x.shape[0] >= tokens
     width = out.shape[1]
     assert y.shape[1] == width and y.dtype == out.dtype and y.shape[0] >= tokens * top and out.shape[0] >= tokens
     assert share.dtype == torch.float32 and share.numel() >= tokens * top
@@ -669,7 +747,7 @@ def moe_combine(y: torch.Tensor, share: torch.Tensor, top: int, shared: torch.Te
         assert shared_gate is None or (shared_gate.dtype == torch.float32 and shared_gate.numel() >= tokens)
     lib.call("dinfer_moe_combine", dtype_code(y.dtype), y.data_ptr(), _rows(y), share.data_ptr(), top, _ptr(shared),
              _rows(shared) if shared is not None else 0, _ptr(shared_gate), out.data_ptr(), _rows(out), tokens, width,
-             _stream())
+             _ptr(idx), int(real_experts), _ptr(x) if idx is not None else 0, _rows(x) if idx is not None else 0, _stream())
     return out
 
 
@@ -714,10 +792,11 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
              positions: torch.Tensor, cos_sin: torch.Tensor | None, rotary_dim: int, rope_style: int,
              k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, slot_mapping: torch.Tensor | None,
              page_size: int, token_runs: bool = True, v_dim: int | None = None, bias: torch.Tensor | None = None,
-             q_temp: tuple | None = None) -> None:
+             q_temp: tuple | None = None, q_head_scale: torch.Tensor | None = None) -> None:
     """Per-head q/k norm, rotation, q written back in place, k and v written to the cache pages.
     bias: float32 [q heads | k heads | v heads], added to the product's output first. q_temp (coef, every): q is
-    multiplied by 1 + coef ln(floor((p + 1) / every) + 1) at position p, together with the norm.
+    multiplied by 1 + coef ln(floor((p + 1) / every) + 1) at position p, together with the norm. q_head_scale: float32
+    [heads], q of head h is multiplied by its entry with the norm (a temperature on the head's scores).
     v_dim: the size of a value head where it is not head_dim. v_cache None beside a k_cache: the values are not stored
     (a layer whose values are its keys reads them from the key pages).
 
@@ -725,7 +804,7 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
     to the cache and k is written back in place, as q is). token_runs: the tokens come in runs of consecutive positions (prompt portions, not
     single decoded tokens); it only chooses the faster of two ways of writing V.
     """
-    _need_gpu(qkv, q_gain, k_gain, positions, cos_sin, k_cache, v_cache, slot_mapping)
+    _need_gpu(qkv, q_gain, k_gain, positions, cos_sin, k_cache, v_cache, slot_mapping, q_head_scale)
     ld = _rows(qkv)
     assert qkv.shape[0] >= tokens
     vd = head_dim if v_dim is None else v_dim
@@ -743,6 +822,8 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
         assert bias.numel() == (heads + kv_heads) * head_dim + kv_heads * vd
     if q_temp is not None:
         assert q_gain is not None and int(q_temp[1]) > 0
+    if q_head_scale is not None:
+        assert q_gain is not None and q_head_scale.dtype == torch.float32 and q_head_scale.numel() == heads
     if slot_mapping is not None:
         assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() >= tokens
         assert k_cache is not None
@@ -752,7 +833,7 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
              _ptr(q_gain), _ptr(k_gain), wf32, float(eps), float(gain_offset), positions.data_ptr(), _ptr(cos_sin),
              rotary_dim, rope_style, _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), heads, kv_heads, head_dim,
              page_size, int(token_runs), vd, _ptr(bias), float(q_temp[0]) if q_temp else 0.0,
-             int(q_temp[1]) if q_temp else 0, _stream())
+             int(q_temp[1]) if q_temp else 0, _ptr(q_head_scale), _stream())
 
 
 def attn_paged_ext(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor | None,
@@ -797,6 +878,29 @@ def attn_paged_ref(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_
              k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
              cu_seqlens.data_ptr(), seq_lens.data_ptr(), num_reqs, tokens, float(scale), int(window), heads,
              kv_heads, head_dim, page_size, _stream())
+    return out
+
+
+def attn_paged_diff(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    block_table: torch.Tensor, cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, num_reqs: int,
+                    tokens: int, *, scale: float, window: int, heads: int, kv_heads: int, head_dim: int, v_dim: int,
+                    page_size: int, lam: float, eps: float, post: float) -> torch.Tensor:
+    """Differential attention, plain kernel: a query head holds two queries of head_dim entries side by side, a key
+    head two keys (pages of heads of 2 head_dim); both softmax attentions run over the same values and
+    out = unit_rms(a1 - lam a2, eps) * post, head h at column h v_dim."""
+    _need_gpu(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens)
+    assert q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
+    assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
+    assert block_table.shape[0] >= num_reqs
+    assert cu_seqlens.dtype == torch.int32 and cu_seqlens.numel() >= num_reqs + 1
+    assert seq_lens.dtype == torch.int32 and seq_lens.numel() >= num_reqs
+    _check_pages(k_cache, v_cache, kv_heads, 2 * head_dim, page_size, v_dim)
+    assert q.shape[1] >= heads * 2 * head_dim and out.shape[1] >= heads * v_dim
+    assert q.shape[0] >= tokens and out.shape[0] >= tokens
+    lib.call("dinfer_attn_paged_diff", dtype_code(q.dtype), q.data_ptr(), _rows(q), out.data_ptr(), _rows(out),
+             k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+             cu_seqlens.data_ptr(), seq_lens.data_ptr(), num_reqs, tokens, float(scale), int(window), heads, kv_heads,
+             head_dim, v_dim, page_size, float(lam), float(eps), float(post), _stream())
     return out
 
 

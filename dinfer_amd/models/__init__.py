@@ -1,1 +1,1 @@
-from . import fanulix, karopel, kudurax, qwen3  # noqa: F401  (register the built-in architectures)
+from . import fanulix, karopel, kudurax, qwen3, verorax  # noqa: F401  (register the built-in architectures)

@@ -13,7 +13,9 @@ values that are the keys (`values_are_keys`: no value projection, no value pages
 root mean square a head without a gain (`qk_unit_eps`); a query that grows with its position, times
 1 + coef ln(floor((p + 1) / every) + 1) (`q_temp = (coef, every)`); a sink of a fixed score instead of a learned one
 (`sink_value`: 0.0 adds one to the softmax's denominator); the concatenated heads multiplied by an activation of one
-more projection of the mixer's input before the output projection (`gate`: "sigmoid" or "silu"). A layer that uses any
+more projection of the mixer's input before the output projection (`gate`: "sigmoid" or "silu"; with `gate_heads` the
+projection gives one number a head, which multiplies all of the head's values); a learned temperature a head that
+multiplies the head's scores (`head_temp`, a tensor [heads]; it rides on the query, in the per-head norm). A layer that uses any
 option runs the flash kernel with options on the matrix cores where its sizes allow, else the plain kernel with options
 (csrc/attention_ref.hip), for prompt portions and single rows alike; the matrix-core kernels serve the others.
 """
@@ -37,14 +39,14 @@ class Attention(Mixer):
 
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "q_norm": "q_norm.", "k_norm": "k_norm.", "sink": "sinks", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias",
-             "v_bias": "v_proj.bias", "g": "g_proj.weight"}
+             "v_bias": "v_proj.bias", "g": "g_proj.weight", "temp": "temp"}
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position: PartSpec,
                  qk_norm: PartSpec | None = None, window: int | None = None, scale: float | None = None,
                  v_dim: int | None = None, keep_first: int = 0, sink: bool = False, slope_exp: float = 0.0,
                  values_are_keys: bool = False, out_scale: float = 1.0, names: dict | None = None, bias: bool = False,
                  qk_unit_eps: float | None = None, q_temp: tuple | None = None, sink_value: float | None = None,
-                 gate: str | None = None):
+                 gate: str | None = None, gate_heads: bool = False, head_temp: bool = False):
         if heads % kv_heads:
             raise ValueError(f"heads {heads} not divisible by kv_heads {kv_heads}")
         if head_dim <= 0 or head_dim > ops.MAX_HEAD_DIM:   # said at build, not at the first step
@@ -73,15 +75,20 @@ class Attention(Mixer):
             raise ValueError("attention: a query temperature needs every > 0 and a per-head norm of q (it rides in it)")
         if gate is not None and gate not in ("sigmoid", "silu"):
             raise ValueError(f"attention: gate {gate!r} unknown (known: 'sigmoid', 'silu')")
+        self.gate_heads, self.head_temp = bool(gate_heads) and gate is not None, bool(head_temp)
+        if self.head_temp and qk_norm is None and qk_unit_eps is None:
+            raise ValueError("attention: a temperature a head needs a per-head norm of q (it rides in it)")
         if self.bias and self.values_are_keys:
             raise ValueError("attention: biases with values that are the keys are not built")
         # what the matrix-core kernels do not do runs through the plain kernel with options
         self.extended = bool(self.v_dim != head_dim or self.keep_first or self.sink or self.slope_exp
                              or self.values_are_keys or self.out_scale != 1.0 or self.bias or qk_unit_eps is not None
-                             or self.q_temp is not None or self.sink_value is not None or gate is not None)
+                             or self.q_temp is not None or self.sink_value is not None or gate is not None
+                             or self.head_temp)
         self.q_size, self.kv_size = heads * head_dim, kv_heads * head_dim
         self.v_size = 0 if self.values_are_keys else kv_heads * self.v_dim
-        self.g_size = heads * self.v_dim if gate is not None else 0
+        self.g_size = (heads if self.gate_heads else heads * self.v_dim) if gate is not None else 0
+        self.temps = None
         self.g_off = self.q_size + self.kv_size + self.v_size
         self.qkv = Linear(hidden, self.q_size + self.kv_size + self.v_size + self.g_size)
         self.bias_vec = self.unit_gain = None
@@ -123,6 +130,8 @@ class Attention(Mixer):
             t[nm["v_bias"]] = TensorSpec((self.v_size,), init="zeros")
         if self.gate is not None:
             t[nm["g"]] = TensorSpec((self.g_size, Hd))
+        if self.head_temp:
+            t[nm["temp"]] = TensorSpec((self.heads,), init="gain")
         for n, spec in self.position.tensors().items():   # an encoding with parameters of its own (rotations have none)
             t["position." + n] = spec
         return t
@@ -166,6 +175,8 @@ class Attention(Mixer):
             self.sinks = torch.full((self.heads,), self.sink_value, dtype=torch.float32, device=some.device)
         if self.bias:     # small parameters in 32 bits (exact for a bfloat16 file): q heads | k heads | v heads
             self.bias_vec = torch.cat([get(nm[k]).float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
+        if self.head_temp:
+            self.temps = get(nm["temp"]).float().contiguous()
         if self.qk_unit_eps is not None:
             self.unit_gain = torch.ones(self.head_dim, dtype=torch.float32, device=some.device)
         self.position.load(lambda n, **kw: get("position." + n, **kw))
@@ -252,11 +263,12 @@ class Attention(Mixer):
                      q_gain=q_gain, k_gain=k_gain, eps=eps, gain_offset=qn.weight_offset if qn else 0.0,
                      cos_sin=pos.table(), rotary_dim=pos.rotary_dim, rope_style=pos.style,
                      k_cache=cache.k, v_cache=cache.v, slot_mapping=batch.slot_mapping[g] if cache.owner else None,
-                     token_runs=False, v_dim=vd, bias=self.bias_vec, q_temp=self.q_temp)
+                     token_runs=False, v_dim=vd, bias=self.bias_vec, q_temp=self.q_temp, q_head_scale=self.temps)
         self._attend_ext(qkv_buf, col, attn_buf, out_col, batch, cache)
         if self.gate is not None:
             n = self.heads * vd
-            ops.gate(attn_buf[:, out_col:out_col + n], qkv_buf[:, col + self.g_off:col + self.g_off + n], T, self.gate)
+            ops.gate(attn_buf[:, out_col:out_col + n], qkv_buf[:, col + self.g_off:col + self.g_off + self.g_size], T,
+                     self.gate, group=vd if self.gate_heads else 1)
 
     def _attend_ext(self, qkv_buf, col, attn_buf, out_col, batch, cache: CacheView):
         T, g, vd = batch.num_tokens, cache.group, self.v_dim

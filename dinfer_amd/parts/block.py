@@ -110,12 +110,19 @@ class SandwichBlock(Block):
     One kernel a sublayer's end norms the branch, adds it into the stream (in the stream's own dtype, 32 bits where
     the model says so) and norms the stream for what reads it next: this block's feed-forward, or the next block's
     mixer (handed over as a Carried that is ready). params: mult, mixer_prefix, ff_prefix and the four norms' names.
-    All four norms are of the layer's norm kind, which must be a root-mean-square norm (`carried()` gives its gain)."""
+    All four norms are of the layer's norm kind, which must be a root-mean-square norm (`carried()` gives its gain).
+
+    shift (a tensor's name, [hidden]): token shift. What the mixer reads, x = norm_a(h), becomes x + (x' - x) * shift,
+    x' the x of the token before in its request as the norm gave it (zeros before the first token). The last x of a
+    request is state of its own, one row a request and run entry, kept beside the mixer's cache: the entry's cache
+    is then the mixer's under "mixer" joined with that row under "shift"."""
     carries_norms = True
 
     def __init__(self, hidden: int, layer: LayerSpec, mult: float = 1.0, mixer_prefix: str = "mix.", ff_prefix: str = "mlp.",
-                 norm_a: str = "norm1", norm_a_out: str = "norm1b", norm_b: str = "norm2", norm_b_out: str = "norm2b"):
+                 norm_a: str = "norm1", norm_a_out: str = "norm1b", norm_b: str = "norm2", norm_b_out: str = "norm2b",
+                 shift: str | None = None):
         self.hidden, self.mult = hidden, float(mult)
+        self.shift_name, self.shift = shift, None
         self.mixer = MIXERS.get(layer.mixer.kind)(hidden=hidden, **layer.mixer.params)
         self.ff = FEED_FORWARDS.get(layer.feed_forward.kind)(hidden=hidden, **layer.feed_forward.params)
         if getattr(self.ff, "absent", False):
@@ -142,18 +149,32 @@ class SandwichBlock(Block):
         return all(part.capturable and part.capturable_portions for _, part in self._parts())
 
     def tensors(self):
-        return {p + n: s for p, part in self._parts() for n, s in part.tensors().items()}
+        t = {p + n: s for p, part in self._parts() for n, s in part.tensors().items()}
+        if self.shift_name is not None:
+            from .spec import TensorSpec
+            t[self.shift_name] = TensorSpec((self.hidden,), init="shares")
+        return t
 
     def load(self, get):
         for p, part in self._parts():
             part.load(_sub(get, p))
         for _, n in self.norms:
             n.weight = n.weight.float().contiguous()     # (exact for a bfloat16 file) one type for all gains of a kernel
+        if self.shift_name is not None:
+            self.shift = get(self.shift_name).float().contiguous()
 
     def bind(self, ctx):
         for _, part in self._parts():
             part.bind(ctx)
         self.normed = ctx.workspace.buffer("normed", self.hidden)
+        if self.shift_name is not None:
+            self.shifted = ctx.workspace.buffer("shifted", self.hidden)
+
+    def cache_spec(self):
+        if self.shift_name is None:
+            return self.mixer.cache_spec()
+        from .spec import JoinedSpec, StateSpec
+        return JoinedSpec({"mixer": self.mixer.cache_spec(), "shift": StateSpec((self.hidden,), dtype="engine")})
 
     def input_norm(self):
         return self.norms[0][1]
@@ -176,6 +197,13 @@ class SandwichBlock(Block):
             if pending is not None:      # a block of another kind left its last branch to be added
                 ops.add_rows(hidden, T, a=pending)
             x = self.norms[0][1].forward(hidden, self.normed, T)
+        if self.shift is not None:
+            if not cache.owner:
+                raise NotImplementedError("token shift keeps a row a request: an entry that borrows a cache has none")
+            x = ops.token_shift(x, self.shifted, cache.child("shift").state, self.shift, cu_seqlens=batch.cu_seqlens,
+                                seq_lens=batch.seq_lens, state_slots=batch.state_slots, num_reqs=batch.num_reqs,
+                                max_rows=batch.max_q_len)
+            cache = cache.child("mixer")
         a = self.mixer.forward(x, batch, cache)
         if next_norm is not None:     # handed on only where the kernel can apply it: a gain of the type of this block's
             params = next_norm.carried()

@@ -15,6 +15,10 @@ qa_h = Wuk_h^T qn_h, s = scale * <[qa_h | qr_h], [c | kr]>, and the attention's 
 by Wuv_h afterwards, so no key or value is ever expanded and prompt portions and single decoded tokens run through
 the same kernels. A layer with `shares_cache` has no down projection: it reads the cache of the run entry it is
 given (written by a layer whose latent sizes and rotation equal its own) with heads, Wuk and Wuv of its own.
+
+With `q_rank` the queries go through a latent of their own: cq = rmsnorm(Wdq h) * wq (the latent norm's kind and eps),
+q = Wuq cq; the first product then makes [cq' | c' | kr'] and a second one the queries (names "dq", "dq.norm", "uq").
+The rotation pairs entries (2i, 2i+1) or (i, i + rot/2), as the position encoding says.
 """
 from __future__ import annotations
 
@@ -36,7 +40,8 @@ class LatentAttention(Mixer):
     def __init__(self, hidden: int, heads: int, dim: int, rot_dim: int, vdim: int, rank: int, scale: float,
                  position: PartSpec, latent_norm: PartSpec, gated: bool = True, shares_cache: bool = False,
                  window: int | None = None,
-                 names: tuple = ("q", "dkv", "dkv.norm", "uk", "uv", "g", "o")):
+                 names: tuple = ("q", "dkv", "dkv.norm", "uk", "uv", "g", "o"), q_rank: int | None = None,
+                 q_names: tuple = ("dq", "dq.norm", "uq")):
         if rank <= 0 or rank > ops.LATENT_MAX_RANK or rank + rot_dim > ops.LATENT_MAX_KEY:
             raise ValueError(f"latent attention: rank {rank} with rot_dim {rot_dim} has no kernel (rank up to "
                              f"{ops.LATENT_MAX_RANK}, rank + rot_dim up to {ops.LATENT_MAX_KEY})")
@@ -44,17 +49,25 @@ class LatentAttention(Mixer):
         self.scale, self.gated, self.shares_cache, self.window = float(scale), gated, shares_cache, window
         self.names = dict(zip(("q", "dkv", "norm", "uk", "uv", "g", "o"), names))
         self.q_size = heads * (dim + rot_dim)
-        self.c_off = None if shares_cache else self.q_size
-        self.g_off = self.q_size + (0 if shares_cache else rank + rot_dim)
+        self.q_rank = int(q_rank) if q_rank else 0
+        self.q_names = dict(zip(("dq", "norm", "uq"), q_names))
+        first = self.q_rank or self.q_size           # what the first product makes of the queries
+        self.c_off = None if shares_cache else first
+        self.g_off = first + (0 if shares_cache else rank + rot_dim)
         used = self.g_off + (heads if gated else 0)
         self.proj = Linear(hidden, -(-used // 8) * 8)      # q | down projection | gate in one product (rows padded to 8)
         self.used = used
         self.o = Linear(heads * vdim, hidden)
         self.position = POSITION_ENCODINGS.get(position.kind)(head_dim=rot_dim, **position.params)
-        if not self.position.fused or (self.position.rotary_dim and self.position.style != 1):
-            raise ValueError("latent attention rotates pairs (2i, 2i+1) by a table: a position encoding of another kind "
-                             "has no kernel here")
+        if not self.position.fused:
+            raise ValueError("latent attention rotates by a table: a position encoding of another kind has no kernel here")
         self.latent_norm = None if shares_cache else NORMS.get(latent_norm.kind)(rank, **latent_norm.params)
+        self.q_norm = self.uq = None
+        if self.q_rank:
+            self.q_norm = NORMS.get(latent_norm.kind)(self.q_rank, **latent_norm.params)
+            self.uq = Linear(self.q_rank, self.q_size)
+            if self.q_norm.carried() is None or self.q_norm.carried()[1] != 0.0:
+                raise ValueError("latent attention norms its query latent by root mean square with a plain gain")
         if self.latent_norm is not None and (self.latent_norm.carried() is None or self.latent_norm.carried()[1] != 0.0):
             raise ValueError("latent attention norms its latent by root mean square with a plain gain")
 
@@ -64,10 +77,17 @@ class LatentAttention(Mixer):
 
     def tensors(self):
         n, H = self.names, self.heads
-        t = {n["q"]: TensorSpec((self.q_size, self.hidden)),
-             n["uk"]: TensorSpec((H * self.dim, self.rank)),
+        t = {n["uk"]: TensorSpec((H * self.dim, self.rank)),
              n["uv"]: TensorSpec((H * self.vdim, self.rank)),
              n["o"]: TensorSpec((self.hidden, H * self.vdim))}
+        if self.q_rank:
+            qn = self.q_names
+            t[qn["dq"]] = TensorSpec((self.q_rank, self.hidden))
+            t[qn["uq"]] = TensorSpec((self.q_size, self.q_rank))
+            for name, spec in self.q_norm.tensors().items():
+                t[qn["norm"] + name] = spec
+        else:
+            t[n["q"]] = TensorSpec((self.q_size, self.hidden))
         if not self.shares_cache:
             t[n["dkv"]] = TensorSpec((self.rank + self.rot_dim, self.hidden))
             for name, spec in self.latent_norm.tensors().items():
@@ -78,7 +98,13 @@ class LatentAttention(Mixer):
 
     def load(self, get):
         n, H = self.names, self.heads
-        rows = [get(n["q"], compute=True)]
+        if self.q_rank:
+            qn = self.q_names
+            rows = [get(qn["dq"], compute=True)]
+            self.q_norm.load(lambda name, **kw: get(qn["norm"] + name, **kw))
+            self.uq.set_weight(get(qn["uq"], compute=True))
+        else:
+            rows = [get(n["q"], compute=True)]
         if not self.shares_cache:
             rows.append(get(n["dkv"], compute=True))
             self.latent_norm.load(lambda name, **kw: get(n["norm"] + name, **kw))
@@ -99,6 +125,9 @@ class LatentAttention(Mixer):
         self.position.bind(ctx)
         H = self.heads
         self.proj_buf = ws.buffer("latent_proj", self.proj.out_features)
+        if self.q_rank:
+            self.cq_buf = ws.buffer("latent_cq", self.q_rank)
+            self.q_buf = ws.buffer("latent_q", self.q_size)
         self.qa_buf = ws.buffer("latent_qa", H * (self.rank + self.rot_dim))
         self.ol_buf = ws.buffer("latent_ol", H * self.rank)
         self.attn_buf = ws.buffer("latent_heads", H * self.vdim)
@@ -111,12 +140,16 @@ class LatentAttention(Mixer):
         self.proj.forward(x, self.proj_buf, T, scratch=True)
         write = cache.owner and not self.shares_cache
         gain = self.latent_norm.weight if write else None
+        q_src = None
+        if self.q_rank:      # the queries' own latent: norm, then the product that makes the queries
+            self.q_norm.forward(self.proj_buf[:, :self.q_rank], self.cq_buf, T)
+            q_src = self.uq.forward(self.cq_buf, self.q_buf, T, scratch=True)
         ops.latent_post(self.proj_buf, T, heads=H, dim=dn, rot_dim=dr, rank=R, q_off=0, c_off=self.c_off if write else None,
                         gain=gain, eps=self.latent_norm.eps if write else 0.0, positions=batch.positions,
                         cos_sin=self.position.table(), rotary_dim=self.position.rotary_dim, qa=self.qa_buf,
                         cache=cache.latent if write else None, slot_mapping=batch.slot_mapping[g] if write else None,
-                        cache_t=cache.tensors.get("latent_t") if write else None)
-        ops.heads_nt(self.proj_buf, 0, dn + dr, self.uk_t, self.qa_buf, 0, R + dr, T)
+                        cache_t=cache.tensors.get("latent_t") if write else None, style=self.position.style, q_src=q_src)
+        ops.heads_nt(self.proj_buf if q_src is None else q_src, 0, dn + dr, self.uk_t, self.qa_buf, 0, R + dr, T)
         latent_kernels.paged_attention(self.qa_buf, self.ol_buf, cache.latent, cache.tensors.get("latent_t"), batch, g,
                                        self.attn_ws, scale=self.scale,
                                        window=self.window or 0, heads=H, rank=R, rot_dim=dr, page_size=self.page_size)

@@ -118,7 +118,10 @@ class DecoderModel:
         """Per run entry: the CacheSpec of the cache it owns; None if it has none or borrows one."""
         out = []
         for i, e in enumerate(self.run):
-            out.append(self.blocks[e.layer].mixer.cache_spec() if e.cache == i else None)
+            block = self.blocks[e.layer]
+            # a block that keeps something of its own between steps answers for its mixer too
+            need = block.cache_spec() if hasattr(block, "cache_spec") else block.mixer.cache_spec()
+            out.append(need if e.cache == i else None)
         return out
 
     def capturable(self) -> bool:

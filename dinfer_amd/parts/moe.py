@@ -9,6 +9,12 @@
 With `gated=False` an expert, and the shared one, is down_e( act(up_e x) ) with act "silu" or "gelu" (error function);
 with `shared_gate=False` the shared expert's output is added as it is.
 
+Another rule of routing (`scores="all"`): the scores are the softmax of z over all router outputs; the `top` largest
+of score + correction are chosen (`correction`, a tensor of one number a router output, only moves the choice), and a
+chosen expert's weight is its score as it is, so a token's weights need not sum to one. `identity` experts: the router
+has `experts + identity` outputs, and the last `identity` of them stand for experts without tensors whose output is
+their input (times the weight).
+
 Per step: one kernel routes (logits, choice, weights, the shared gate), one sorts the (token, choice) entries by
 expert and writes the work list of row tiles, two launches run the products of all experts (gate and up with the
 activation, then down, each row computed alone and written to its entry's place), and one sums a token's entries in
@@ -33,12 +39,18 @@ class RoutedExperts(FeedForward):
     [1, hidden] where `shared_intermediate` is given."""
 
     def __init__(self, hidden: int, experts: int, top: int, intermediate: int, shared_intermediate: int | None = None,
-                 act: str = "silu", gated: bool = True, shared_gate: bool = True):
+                 act: str = "silu", gated: bool = True, shared_gate: bool = True, scores: str = "chosen",
+                 correction: bool = False, identity: int = 0):
         if gated and act != "silu":
             raise ValueError(f"routed feed-forward: gated activation {act!r} has no kernel (known: ['silu'])")
         if not gated and act not in ops.EXPERT_ACTS:
             raise ValueError(f"routed feed-forward: activation {act!r} has no kernel (known: {sorted(ops.EXPERT_ACTS)})")
-        if not (0 < top <= experts) or experts > ops.MOE_MAX_EXPERTS or top > ops.MOE_MAX_TOP:
+        if scores not in ("chosen", "all") or identity < 0 or (scores != "all" and (correction or identity)):
+            raise ValueError(f"routed feed-forward: scores {scores!r} with correction {correction} and {identity} identity "
+                             "experts: a correction and identity experts go with scores over all router outputs")
+        self.all_scores, self.has_correction, self.identity = scores == "all", bool(correction), int(identity)
+        self.outputs = experts + self.identity          # what the router gives a token
+        if not (0 < top <= self.outputs) or self.outputs > ops.MOE_MAX_EXPERTS or top > ops.MOE_MAX_TOP:
             raise ValueError(f"routed feed-forward: {top} of {experts} experts has no kernel (up to {ops.MOE_MAX_TOP} of "
                              f"{ops.MOE_MAX_EXPERTS})")
         self.hidden, self.experts, self.top, self.intermediate = hidden, experts, top, intermediate
@@ -52,7 +64,9 @@ class RoutedExperts(FeedForward):
                               act_name="shared_act")
 
     def tensors(self):
-        t = {"router": TensorSpec((self.experts, self.hidden))}
+        t = {"router": TensorSpec((self.outputs, self.hidden))}
+        if self.has_correction:
+            t["correction"] = TensorSpec((self.outputs,), init="zeros")
         for e in range(self.experts):
             if self.gated:
                 t[f"e{e}.gate"] = TensorSpec((self.intermediate, self.hidden))
@@ -66,6 +80,7 @@ class RoutedExperts(FeedForward):
 
     def load(self, get):
         self.router = get("router").float().contiguous()       # routing runs in 32 bits
+        self.correction = get("correction").float().contiguous() if self.has_correction else None
         E = range(self.experts)
         # [experts, 2 I, hidden]: an expert's gate rows, then its up rows (not gated: [experts, I, hidden]); [experts, hidden, I]
         if self.gated:
@@ -86,12 +101,12 @@ class RoutedExperts(FeedForward):
         i32 = torch.int32
         self.idx = torch.zeros(n, dtype=i32, device=dev)
         self.share = torch.zeros(n, dtype=torch.float32, device=dev)
-        self.logits = torch.zeros(ctx.max_tokens * (self.experts + 1), dtype=torch.float32, device=dev)
+        self.logits = torch.zeros(ctx.max_tokens * (self.outputs + 1), dtype=torch.float32, device=dev)
         self.shared_gate = torch.zeros(ctx.max_tokens, dtype=torch.float32, device=dev)
-        self.offsets = torch.zeros(self.experts + 1, dtype=i32, device=dev)
+        self.offsets = torch.zeros(self.outputs + 1, dtype=i32, device=dev)
         self.perm = torch.zeros(n, dtype=i32, device=dev)
         self.dtype = ctx.dtype
-        self.tiles = torch.zeros((ops.moe_max_tiles(n, self.experts, 16), 2), dtype=i32, device=dev)   # the smallest tile: the longest list
+        self.tiles = torch.zeros((ops.moe_max_tiles(n, self.outputs, 16), 2), dtype=i32, device=dev)   # the smallest tile: the longest list
         self.act_buf = ws.buffer("moe_act", self.intermediate, rows=n)
         self.y_buf = ws.buffer("moe_y", self.hidden, rows=n)
         self.out_buf = ws.buffer("ffn_out", self.hidden)
@@ -101,13 +116,15 @@ class RoutedExperts(FeedForward):
     def forward(self, x, batch, into=None):
         T, top = batch.num_tokens, self.top
         n = T * top
-        ops.moe_route(x, self.router, self.sg, self.idx, self.share, self.shared_gate, T, top, self.logits)
-        rows = ops.moe_tile_rows(self.dtype, n, self.experts, self.hidden, self.intermediate)   # follows the step's count alone
-        ops.moe_scatter(self.idx, n, self.experts, self.offsets, self.perm, self.tiles, rows)
+        ops.moe_route(x, self.router, self.sg, self.idx, self.share, self.shared_gate, T, top, self.logits,
+                      all_scores=self.all_scores, correction=self.correction)
+        rows = ops.moe_tile_rows(self.dtype, n, self.outputs, self.hidden, self.intermediate)   # follows the step's count alone
+        ops.moe_scatter(self.idx, n, self.outputs, self.offsets, self.perm, self.tiles, rows, real_experts=self.experts)
         ops.experts_nt(x, self.w_in, self.act_buf, n, self.tiles, self.offsets, self.perm, gated=self.gated, a_div=top,
                        c_to_perm=False, tile_rows=rows, act=None if self.gated else self.act)
         ops.experts_nt(self.act_buf, self.w_out, self.y_buf, n, self.tiles, self.offsets, self.perm, gated=False, a_div=0,
                        c_to_perm=True, tile_rows=rows)
         shared = self.shared.forward(x, batch) if self.shared is not None else None
+        same = dict(idx=self.idx, real_experts=self.experts, x=x) if self.identity else {}
         return ops.moe_combine(self.y_buf, self.share, top, shared, self.shared_gate if self.sg is not None else None,
-                               self.out_buf, T)
+                               self.out_buf, T, **same)

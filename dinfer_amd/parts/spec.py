@@ -30,7 +30,7 @@ class TensorSpec:
     """One tensor a part expects from the weight file.
 
     init: how the random-weights mode draws it: "linear" N(0, 0.02), "gain"
-    1 + N(0, 0.1), "zeros", "ones", "eye" (the unit matrix). keep_f32: stays 32-bit even in a bfloat16
+    1 + N(0, 0.1), "shares" uniform in [0, 1), "zeros", "ones", "eye" (the unit matrix). keep_f32: stays 32-bit even in a bfloat16
     engine when the file stores it so.
     """
     shape: tuple
@@ -146,21 +146,25 @@ class LatentSpec(CacheSpec):
 @dataclass(frozen=True)
 class StateSpec(CacheSpec):
     """Cache need of a mixer with per-request state of fixed size (shape per request). The state cannot be rebuilt
-    from pages, so a model that has one gets no prefix cache."""
+    from pages, so a model that has one gets no prefix cache. dtype: a torch dtype's name, or "engine" for the dtype
+    the engine computes in."""
     shape: tuple
     dtype: str = "float32"
     recomputable = False
 
-    def slot_bytes(self, dtype):
+    def _dtype(self, engine_dtype):
         import torch
+        return engine_dtype if self.dtype == "engine" else getattr(torch, self.dtype)
+
+    def slot_bytes(self, dtype):
         n = 1
         for s in self.shape:
             n *= s
-        return n * _element_size(getattr(torch, self.dtype))
+        return n * _element_size(self._dtype(dtype))
 
     def allocate(self, num_blocks, page_size, num_slots, dtype, device):
         import torch
-        return {"state": torch.zeros((num_slots, *self.shape), dtype=getattr(torch, self.dtype), device=device)}
+        return {"state": torch.zeros((num_slots, *self.shape), dtype=self._dtype(dtype), device=device)}
 
     def reset_slots(self, tensors, slots):
         tensors["state"].index_fill_(0, slots, 0)

@@ -35,6 +35,8 @@ def draw(seed: int, name: str, spec: TensorSpec, dtype: torch.dtype) -> torch.Te
         t = torch.randn(spec.shape, generator=g, dtype=torch.float32) * LINEAR_STD
     elif spec.init == "gain":
         t = 1.0 + torch.randn(spec.shape, generator=g, dtype=torch.float32) * GAIN_STD
+    elif spec.init == "shares":
+        t = torch.rand(spec.shape, generator=g, dtype=torch.float32)
     elif spec.init == "zeros":
         t = torch.zeros(spec.shape, dtype=torch.float32)
     elif spec.init == "ones":
@@ -54,6 +56,8 @@ def draw_on_device(seed: int, name: str, spec: TensorSpec, dtype: torch.dtype, d
         return draw(seed, name, spec, dtype).to(device)
     g = torch.Generator(device=device)
     g.manual_seed(tensor_seed(seed, name))
+    if spec.init == "shares":
+        return torch.rand(spec.shape, generator=g, device=device, dtype=torch.float32).to(dtype)
     t = torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)
     if spec.init == "linear":
         t *= LINEAR_STD

@@ -133,6 +133,18 @@ class SafetensorsDir:
             f.fh.close()
 
 
+def tensor_shapes(model_dir: str | Path) -> dict:
+    """name -> shape of every tensor in the folder's *.safetensors, from their headers alone; {} where there is no
+    such file (a configuration that is read without its weights)."""
+    if not list(Path(model_dir).glob("*.safetensors")):
+        return {}
+    d = SafetensorsDir(model_dir)
+    try:
+        return {n: ti.shape for n, ti in d.index.items()}
+    finally:
+        d.close()
+
+
 def write_safetensors(path: str | Path, tensors: dict[str, torch.Tensor], metadata: dict | None = None) -> None:
     """Writes one file; tensors in name order, data 8-byte aligned after the header."""
     header = {}
