@@ -159,16 +159,31 @@ def dense_ff(h, w, p):
     return (gelu_tanh(h @ w[p + ".gate"].T) * (h @ w[p + ".up"].T)) @ w[p + ".down"].T
 
 
-def chosen_experts(h, w, p, f):
-    """(indices [T, top], weights [T, top]): softmax over all router outputs; the correction only moves the choice."""
+CLOSE_CALL = 0.05     # choice scores nearer than this may fall either way once the router's input is rounded
+
+
+def chosen_experts(h, w, p, f, given=None):
+    """(indices [T, top], weights [T, top]): softmax over all router outputs; the correction only moves the choice.
+    given {row: [experts]}: the choice somebody else made for some rows (an engine whose router read rounded rows). It
+    is taken over where it could be right: every expert it names scores within CLOSE_CALL of the last one chosen here,
+    and every expert chosen here that it leaves out is within CLOSE_CALL of the best one it could have left out."""
+    top = f["router"]["top"]
     s = torch.softmax(h @ w[p + ".router"].T, dim=-1)
-    idx = torch.topk(s + w[p + ".correction"], f["router"]["top"], dim=-1).indices
+    choice = s + w[p + ".correction"]
+    idx = torch.topk(choice, top, dim=-1).indices
+    for t, other in (given or {}).items():
+        assert len(other) == top == len(set(other)), f"{p} row {t}: {other} are not {top} experts"
+        line = choice[t, idx[t]].min().item()
+        assert all(choice[t, e].item() > line - CLOSE_CALL for e in other), f"{p} row {t}: {other} chosen, {idx[t].tolist()} score best"
+        assert all(choice[t, e].item() < line + CLOSE_CALL for e in idx[t].tolist() if e not in other), \
+            f"{p} row {t}: {other} chosen, {idx[t].tolist()} score best"
+        idx[t] = torch.tensor(other)
     return idx, torch.gather(s, 1, idx)
 
 
-def routed_ff(h, w, p, f):
+def routed_ff(h, w, p, f, given=None):
     E = f["router"]["experts"]
-    idx, share = chosen_experts(h, w, p, f)
+    idx, share = chosen_experts(h, w, p, f, given)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, s in zip(idx[t].tolist(), share[t]):
@@ -183,8 +198,9 @@ def routed_ff(h, w, p, f):
 MIXERS = {"latent_attention": latent_attention, "attention": differential_attention, "parallel": parallel}
 
 
-def layer(x, w, cfg, i):
-    """One entry of the layer list on the stream x [T, width]; an entry with weights_of reads that layer's tensors."""
+def layer(x, w, cfg, i, given=None):
+    """One entry of the layer list on the stream x [T, width]; an entry with weights_of reads that layer's tensors.
+    given: see chosen_experts."""
     l = cfg["layers"][i]
     p = f"l{l.get('weights_of', i)}"
     eps = cfg["norm"]["eps"]
@@ -193,16 +209,101 @@ def layer(x, w, cfg, i):
     f = l.get("mlp")
     if f is not None:
         h = norm(x, w[p + ".norm2"], eps)
-        y = dense_ff(h, w, p + ".mlp") if f["kind"] == "dense" else routed_ff(h, w, p + ".mlp", f)
+        y = dense_ff(h, w, p + ".mlp") if f["kind"] == "dense" else routed_ff(h, w, p + ".mlp", f, given)
         x = x + norm(y, w[p + ".norm2b"], eps)
     return x
 
 
-def forward(tokens, w, cfg, streams=None):
-    """Logits [T, vocab] of a whole sequence; `streams`, a list, receives the stream after every layer."""
+def forward(tokens, w, cfg, streams=None, choices=None):
+    """Logits [T, vocab] of a whole sequence; `streams`, a list, receives the stream after every layer.
+    choices {(layer, row): [experts]}: routing choices to take over where they could be right (chosen_experts)."""
     x = w["embed"][torch.as_tensor(tokens)]
     for i in range(len(cfg["layers"])):
-        x = layer(x, w, cfg, i)
+        x = layer(x, w, cfg, i, {t: e for (l, t), e in (choices or {}).items() if l == i})
         if streams is not None:
             streams.append(x)
     return norm(x, w["final.norm"], cfg["norm"]["eps"]) @ w["head"].T
+
+
+# ---- made-up weights for the tests -------------------------------------------------------------------------------
+def tensor_shapes(cfg, low=6):
+    """name -> shape of every tensor a configuration asks for; `low`: the inner size of the decay projections (the
+    configuration does not hold it: the engine reads it off the tensor)."""
+    W, out = cfg["width"], {"embed": (cfg["vocab"], cfg["width"]), "final.norm": (cfg["width"],), "head": (cfg["vocab"], cfg["width"])}
+    for i, l in enumerate(cfg["layers"]):
+        if "weights_of" in l:
+            continue
+        p, m = f"l{i}", l["mixer"]
+        for n in ("norm1", "norm1b", "shift"):
+            out[f"{p}.{n}"] = (W,)
+        if l["type"] == "latent_attention":
+            H, dn, dr, dv, R, Q = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            out.update({f"{p}.mix.dq": (Q, W), f"{p}.mix.dq.norm": (Q,), f"{p}.mix.uq": (H * (dn + dr), Q),
+                        f"{p}.mix.dkv": (R + dr, W), f"{p}.mix.dkv.norm": (R,), f"{p}.mix.uk": (H * dn, R),
+                        f"{p}.mix.uv": (H * dv, R), f"{p}.mix.o": (W, H * dv)})
+        elif l["type"] == "attention":
+            H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            out.update({f"{p}.mix.q": (2 * H * D, W), f"{p}.mix.q.b": (2 * H * D,), f"{p}.mix.k": (2 * G * D, W),
+                        f"{p}.mix.k.b": (2 * G * D,), f"{p}.mix.v": (G * V, W), f"{p}.mix.v.b": (G * V,),
+                        f"{p}.mix.o": (W, H * V)})
+            for n in ("lq1", "lk1", "lq2", "lk2"):
+                out[f"{p}.mix.{n}"] = (D,)
+        else:
+            a, r = m["left"], m["right"]
+            H, G, D, V = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            out.update({f"{p}.mix.left.q": (H * D, W), f"{p}.mix.left.k": (G * D, W), f"{p}.mix.left.v": (G * V, W),
+                        f"{p}.mix.left.q.norm": (D,), f"{p}.mix.left.k.norm": (D,), f"{p}.mix.left.temp": (H,),
+                        f"{p}.mix.left.g": (H, W), f"{p}.mix.left.o": (W, H * V)})
+            s = r["heads"] * r["dim"]
+            rank = r.get("decay_rank", low)
+            for n in ("r", "k", "v", "g", "a"):
+                out[f"{p}.mix.right.{n}"] = (s, W)
+            out.update({f"{p}.mix.right.a.b": (s,), f"{p}.mix.right.w1": (rank, W), f"{p}.mix.right.w2": (s, rank),
+                        f"{p}.mix.right.w0": (s,), f"{p}.mix.right.norm": (s,), f"{p}.mix.right.o": (W, s)})
+        f = l.get("mlp")
+        if f is not None:
+            out[f"{p}.norm2"] = out[f"{p}.norm2b"] = (W,)
+            if f["kind"] == "dense":
+                out.update({f"{p}.mlp.gate": (f["ff"], W), f"{p}.mlp.up": (f["ff"], W), f"{p}.mlp.down": (W, f["ff"])})
+            else:
+                E, n = f["router"]["experts"], f["router"]["experts"] + f["router"].get("identity", 0)
+                out.update({f"{p}.mlp.router": (n, W), f"{p}.mlp.correction": (n,)})
+                for e in range(E):
+                    I = f["expert"]["ff"]
+                    out.update({f"{p}.mlp.e{e}.gate": (I, W), f"{p}.mlp.e{e}.up": (I, W), f"{p}.mlp.e{e}.down": (W, I)})
+    return out
+
+
+def random_weights(cfg, seed, low=6):
+    """bfloat16 tensors of sizes that keep every mechanism awake: products of unit spread, gains around one, shares
+    between 0 and 1, router corrections large enough to change choices, decay and removal parameters spread over a
+    few units."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg, low).items():
+        last = name.split(".")[-1]
+        x = torch.randn(shape, generator=g)
+        if name == "embed":
+            t = x
+        elif last == "shift":
+            t = torch.rand(shape, generator=g)
+        elif last in ("norm1", "norm1b", "norm2", "norm2b", "norm", "temp"):
+            t = 1.0 + x * 0.2
+        elif last == "correction":
+            t = x * 0.1
+        elif last == "router":
+            t = x * (3.0 / shape[-1] ** 0.5)
+        elif last in ("w0", "b"):
+            t = x * 0.8
+        elif last in ("lq1", "lk1", "lq2", "lk2"):
+            t = x * 0.3
+        elif last == "w2":
+            t = x * (2.5 / shape[-1] ** 0.5)
+        else:
+            t = x * (1.5 / shape[-1] ** 0.5)
+        out[name] = t.to(torch.bfloat16)
+    return out
+
+
+def as_float64(w):
+    return {k: v.to(F) for k, v in w.items()}
