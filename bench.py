@@ -7,6 +7,7 @@
     python bench.py --workload kudurax [--kudurax-shape 2k|4k] [--layers 4] [--prompt 2048] [--only kudurax|qwen3]
     python bench.py --workload karopel [--karopel-shape 2k|4k] [--layers 4] [--prompt 2048] [--only karopel|qwen3]
     python bench.py --workload fanulix [--fanulix-shape 2k|4k] [--layers 4] [--prompt 2048] [--only fanulix|karopel|qwen3]
+    python bench.py --workload verorax [--verorax-shape 2k|4k] [--layers 4] [--prompt 2048] [--only verorax|kudurax|karopel|qwen3]
 
 Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
 request with a 2,048-token prompt in a 4,096-token context; a "step" is one decode step
@@ -287,6 +288,63 @@ def fanulix_config(shape: dict, layers: int, vocab: int) -> dict:
                 norm=dict(eps=1e-5), layers=[ssm if i % 4 == 1 else par for i in range(layers)])
 
 
+# Verorax layer sizes that resemble a real model's: latent attention of 512 + 64 a token with queries through a latent
+# of 1,536; a differential attention of heads of two maps of 64 over values of 128, a window of 1,024; a gated
+# attention with a window of 512 and half of each head rotated beside a delta rule with per-channel decay (heads of 64,
+# a decay projection of 64 inside); dense gelu feed-forwards and 64 routed experts plus 2 identity experts of which a
+# token uses 6. Beside them Kudurax layers (latent attention, routed experts) and Karopel layers (norms on both sides,
+# an attention beside a delta rule) of the same width, and Qwen3 layers
+VERORAX_SHAPES = {
+    "2k": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, rank=512, q_rank=1536, diff_heads=16, diff_kv_heads=4,
+               diff_dim=64, diff_vdim=128, window=1024, left_heads=8, left_kv_heads=2, left_window=512, left_rot=64,
+               delta_heads=32, delta_dim=64, decay_rank=64, ff=8192, experts=64, identity=2, top=6, expert_ff=1408,
+               kudurax="2k", karopel="2k",
+               qwen=dict(num_attention_heads=16, num_key_value_heads=4, head_dim=128, intermediate_size=8192)),
+    "4k": dict(width=4096, heads=32, dim=128, rot_dim=64, vdim=128, rank=512, q_rank=1536, diff_heads=32, diff_kv_heads=8,
+               diff_dim=64, diff_vdim=128, window=1024, left_heads=16, left_kv_heads=4, left_window=512, left_rot=64,
+               delta_heads=64, delta_dim=64, decay_rank=64, ff=12288, experts=64, identity=2, top=8, expert_ff=1536,
+               kudurax="4k", karopel="4k",
+               qwen=dict(num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288)),
+}
+
+
+def verorax_config(shape: dict, layers: int, vocab: int) -> dict:
+    """Layers in fours: latent attention (dense), latent attention, differential attention, parallel (routed); with
+    eight layers or more the last runs on the weights of the fourth."""
+    d = shape["dim"]
+    dense = dict(kind="dense", ff=shape["ff"])
+    moe = dict(kind="moe", expert=dict(ff=shape["expert_ff"]),
+               router=dict(experts=shape["experts"], identity=shape["identity"], top=shape["top"]))
+    lat = dict(heads=shape["heads"], dim=d, rot_dim=shape["rot_dim"], vdim=shape["vdim"], kv_rank=shape["rank"],
+               q_rank=shape["q_rank"], scale=(d + shape["rot_dim"]) ** -0.5, rot=dict(base=10000.0, dims=shape["rot_dim"]))
+    dif = dict(heads=shape["diff_heads"], kv_heads=shape["diff_kv_heads"], dim=shape["diff_dim"], vdim=shape["diff_vdim"],
+               scale=shape["diff_dim"] ** -0.5, diff=0.3, mask=dict(size=shape["window"]))
+    par = dict(left=dict(heads=shape["left_heads"], kv_heads=shape["left_kv_heads"], dim=d, vdim=d, scale=d ** -0.5,
+                         mask=dict(size=shape["left_window"]), rot=dict(base=1000000.0, dims=shape["left_rot"])),
+               right=dict(heads=shape["delta_heads"], dim=shape["delta_dim"], decay_rank=shape["decay_rank"]),
+               left_scale=0.5, right_scale=0.5)
+    four = [dict(type="latent_attention", mixer=lat, mlp=dense), dict(type="latent_attention", mixer=lat, mlp=moe),
+            dict(type="attention", mixer=dif, mlp=moe), dict(type="parallel", mixer=par, mlp=moe)]
+    out = [dict(four[i % 4]) for i in range(layers)]
+    if layers >= 8:
+        out[-1] = dict(out[3], weights_of=3) if (layers - 1) % 4 == 3 else out[-1]
+    return dict(architecture="Verorax", vocab=vocab, width=shape["width"], norm=dict(eps=1e-5), layers=out)
+
+
+def verorax(a, torch, Engine, SamplingParams) -> int:
+    """Prefill and decode throughput of Verorax layers of a real model's sizes beside Kudurax, Karopel and Qwen3 layers of
+    the same width."""
+    from dinfer_amd.config.karopel import KaropelConfig
+    from dinfer_amd.config.kudurax import KuduraxConfig
+    from dinfer_amd.config.verorax import VeroraxConfig
+    shape = VERORAX_SHAPES[a.verorax_shape]
+    layers = a.layers or 4
+    beside = {"kudurax": KuduraxConfig.from_dict(kudurax_config(KUDURAX_SHAPES[shape["kudurax"]], layers, 32768)),
+              "karopel": KaropelConfig.from_dict(karopel_config(KAROPEL_SHAPES[shape["karopel"]], layers, 32768))}
+    return beside_qwen3(a, torch, Engine, SamplingParams, "verorax", "Verorax", a.verorax_shape, shape,
+                        VeroraxConfig.from_dict(verorax_config(shape, layers, 32768)), beside=beside)
+
+
 def fanulix(a, torch, Engine, SamplingParams) -> int:
     """Prefill and decode throughput of Fanulix layers of a real model's sizes beside Karopel and Qwen3 layers of the same
     width."""
@@ -406,9 +464,10 @@ def main() -> int:
     ap.add_argument("--kudurax-shape", default="2k", choices=sorted(KUDURAX_SHAPES), help="kudurax: layer sizes")
     ap.add_argument("--karopel-shape", default="2k", choices=sorted(KAROPEL_SHAPES), help="karopel: layer sizes")
     ap.add_argument("--fanulix-shape", default="2k", choices=sorted(FANULIX_SHAPES), help="fanulix: layer sizes")
-    ap.add_argument("--only", default="", choices=["", "kudurax", "karopel", "fanulix", "qwen3"],
+    ap.add_argument("--verorax-shape", default="2k", choices=sorted(VERORAX_SHAPES), help="verorax: layer sizes")
+    ap.add_argument("--only", default="", choices=["", "kudurax", "karopel", "fanulix", "verorax", "qwen3"],
                     help="kudurax, karopel, fanulix: measure one of the models")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed", "kudurax", "karopel", "fanulix"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed", "kudurax", "karopel", "fanulix", "verorax"],
                     help="serving: 32 requests with prompts of 512 to 3,072 tokens fed in portions of 512 beside the "
                          "requests that decode, 256 outputs each (meant for the 14B shape); closed: --concurrency "
                          "requests live at any time, --prompt tokens in and --max-tokens out each, the load of the "
@@ -434,6 +493,8 @@ def main() -> int:
         return kudurax(a, torch, Engine, SamplingParams)
     if a.workload == "karopel":
         return karopel(a, torch, Engine, SamplingParams)
+    if a.workload == "verorax":
+        return verorax(a, torch, Engine, SamplingParams)
     if a.workload == "fanulix":
         return fanulix(a, torch, Engine, SamplingParams)
     if a.workload == "serving":

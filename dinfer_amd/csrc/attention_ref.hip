@@ -243,6 +243,35 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_diff_kernel(
   }
 }
 
+// The end of a differential head where its two maps were computed as heads of their own (side by side, the first map's
+// Dv values and then the second's): o = a1 - lambda a2, o <- o / sqrt(mean(o^2) + eps) * post. One wave per (token, head).
+template <class S>
+__global__ void __launch_bounds__(WAVES * 64) diff_combine_kernel(const S* __restrict__ in, int64_t ld_in, S* __restrict__ out,
+                                                                  int64_t ld_out, int H, int Dv, float lambda, float eps,
+                                                                  float post) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * WAVES + wave;
+  if (h >= H) return;
+  const S* a = in + (int64_t)t * ld_in + (int64_t)2 * h * Dv;
+  constexpr int NC = MAX_D / 64;
+  float o[NC];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int d = lane + 64 * c;
+    o[c] = d < Dv ? to_f32(a[d]) - lambda * to_f32(a[Dv + d]) : 0.f;
+    ss += o[c] * o[c];
+  }
+  const float inv = post / sqrtf(wave_sum(ss) / (float)Dv + eps);
+  S* orow = out + (int64_t)t * ld_out + (int64_t)h * Dv;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int d = lane + 64 * c;
+    if (d < Dv) orow[d] = from_f32<S>(o[c] * inv);
+  }
+}
+
 }  // namespace
 
 // q [T, ld_q] (head h at column h*D), out [T, ld_out]; block_table [num_reqs, max_blocks];
@@ -308,6 +337,21 @@ extern "C" int dinfer_attn_paged_diff(int dtype, const void* q, int64_t ld_q, vo
     attn_paged_diff_kernel<S><<<grid, WAVES * 64, 0, stream>>>(
         (const S*)q, ld_q, (S*)out, ld_out, (const S*)k_cache, (const S*)v_cache, block_table, max_blocks, cu_seqlens,
         seq_lens, num_reqs, scale, window, heads, kv_heads, head_dim, page_size, v_dim, lambda, eps, post);
+  });
+  return launch_status();
+}
+
+// in [T, ld_in]: head h's two maps at columns 2 h v_dim and (2 h + 1) v_dim; out [T, ld_out]: head h at h v_dim.
+extern "C" int dinfer_diff_combine(int dtype, const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t tokens,
+                                   int heads, int v_dim, float lambda, float eps, float post, hipStream_t stream) {
+  if (tokens <= 0) return OK;
+  if (heads <= 0 || v_dim <= 0 || tokens > 0x7fffffff || ld_in < 2LL * heads * v_dim || ld_out < (int64_t)heads * v_dim)
+    return ERR_BAD_SHAPE;
+  if (v_dim > MAX_D) return ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)tokens, (unsigned)((heads + WAVES - 1) / WAVES));
+  DINFER_DISPATCH_DTYPE(dtype, {
+    diff_combine_kernel<S><<<grid, WAVES * 64, 0, stream>>>((const S*)in, ld_in, (S*)out, ld_out, heads, v_dim, lambda, eps,
+                                                            post);
   });
   return launch_status();
 }

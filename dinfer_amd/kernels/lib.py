@@ -56,6 +56,7 @@ SIGNATURES = {
         "attention_ref",
         [_I, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P],
     ),
+    "dinfer_diff_combine": ("attention_ref", [_I, _P, _L, _P, _L, _L, _I, _I, _F, _F, _F, _P]),
     "dinfer_rmsnorm_stream": ("norm", [_P, _I, _L, _P, _F, _F, _F, _P, _I, _L, _P, _P, _I, _P, _I, _F, _F, _L, _L, _P]),
     "dinfer_axpby": ("elementwise", [_I, _P, _L, _F, _P, _L, _F, _P, _L, _L, _L, _P]),
     "dinfer_add_rows": ("elementwise", [_P, _I, _L, _P, _I, _L, _P, _I, _L, _L, _P]),

@@ -904,6 +904,18 @@ def attn_paged_diff(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v
     return out
 
 
+def diff_combine(pairs: torch.Tensor, out: torch.Tensor, tokens: int, *, heads: int, v_dim: int, lam: float, eps: float,
+                 post: float) -> torch.Tensor:
+    """The end of differential heads whose two maps were computed as heads of their own: pairs [T, 2 heads v_dim]
+    (a head's first map, then its second) -> out[t, h] = unit_rms(a1 - lam a2, eps) * post."""
+    _need_gpu(pairs, out)
+    assert pairs.dtype == out.dtype and pairs.shape[1] >= 2 * heads * v_dim and out.shape[1] >= heads * v_dim
+    assert pairs.shape[0] >= tokens and out.shape[0] >= tokens
+    lib.call("dinfer_diff_combine", dtype_code(out.dtype), pairs.data_ptr(), _rows(pairs), out.data_ptr(), _rows(out), tokens,
+             heads, v_dim, float(lam), float(eps), float(post), _stream())
+    return out
+
+
 def attn_mfma_supports(head_dim: int, page_size: int, heads: int, kv_heads: int) -> bool:
     return bool(lib.get("dinfer_attn_mfma_supports")(head_dim, page_size, heads, kv_heads))
 

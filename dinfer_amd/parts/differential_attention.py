@@ -11,8 +11,15 @@ map's queries and keys, V the value size:
     y = Wo concat_h(o_h)
 
 No positions enter the scores. The cache holds, a token and key/value head, the two keys side by side (a key head of
-2 D entries in the key pages) and the value. One kernel walks the keys once for both maps (csrc/attention_ref.hip);
-prompt portions and single rows run the same kernel.
+2 D entries in the key pages) and the value. The plain kernel walks the keys once for both maps
+(csrc/attention_ref.hip); prompt portions and single rows run the same kernel.
+
+On the matrix cores (bfloat16, V = 2 D, sizes the flash kernel takes): a map is a query head of its own, 2 D wide, whose
+other map's half is zero, [q_1 | 0] and [0 | q_2]; against the key head [k_1 | k_2] it scores q_m . k_m, and the 2 H
+such heads over G key/value heads are grouped-query attention as the flash kernel with options runs it (the zeros come
+out of the projection: the rows of Wq and bq are spread at bind). A small kernel then takes lambda times the second
+map off the first and norms (csrc/attention_ref.hip, diff_combine). The products with the zeros are a third more
+arithmetic than the maps need and run an order of magnitude faster than the plain kernel's.
 """
 from __future__ import annotations
 
@@ -50,6 +57,7 @@ class DifferentialAttention(Mixer):
         self.o = Linear(heads * vdim, hidden)
         self.bias_vec = None
         self.lam = 0.0
+        self.mfma = False      # decided in bind
 
     def cache_spec(self):
         return KVSpec(self.kv_heads, 2 * self.dim, self.window, v_dim=self.vdim)
@@ -66,6 +74,16 @@ class DifferentialAttention(Mixer):
             t[n[k]] = TensorSpec((self.dim,))
         return t
 
+    def _spread(self, q: torch.Tensor) -> torch.Tensor:
+        """Rows (or entries) of the queries [H, 2, D, ...] -> [H, 2, 2 D, ...]: map m keeps its place in a head of 2 D,
+        the other map's half is zero."""
+        H, D = self.heads, self.dim
+        q = q.view(H, 2, D, *q.shape[1:])
+        out = q.new_zeros((H, 2, 2 * D, *q.shape[3:]))
+        out[:, 0, :D] = q[:, 0]
+        out[:, 1, D:] = q[:, 1]
+        return out.view(H * 4 * D, *q.shape[3:])
+
     def load(self, get):
         n = self.names
         self.qkv.set_weight(torch.cat([get(n[k], compute=True) for k in ("q", "k", "v")], dim=0))
@@ -78,6 +96,16 @@ class DifferentialAttention(Mixer):
     def bind(self, ctx):
         ws = ctx.workspace
         self.page_size = ctx.page_size
+        self.mfma = bool(ctx.dtype == torch.bfloat16 and self.vdim == 2 * self.dim
+                         and ops.attn_mfma_supports(2 * self.dim, ctx.page_size, 2 * self.heads, self.kv_heads))
+        if self.mfma and self.qkv.out_features == self.q_size + self.k_size + self.v_size:
+            # every map a query head of its own (see the top): the projection makes the zeros
+            w, q = self.qkv.weight, self.q_size
+            self.qkv = Linear(self.hidden, 2 * q + self.k_size + self.v_size)
+            self.qkv.set_weight(torch.cat([self._spread(w[:q]), w[q:]], dim=0))
+            if self.bias_vec is not None:
+                self.bias_vec = torch.cat([self._spread(self.bias_vec[:q]), self.bias_vec[q:]]).contiguous()
+            self.pair_buf = ws.buffer("diff_pairs", 2 * self.heads * self.vdim)
         self.qkv_buf = ws.buffer("qkv", self.qkv.out_features)
         self.attn_buf = ws.buffer("attn", self.heads * self.vdim)
         self.out_buf = ws.buffer("mixer_out", self.hidden)
@@ -85,13 +113,23 @@ class DifferentialAttention(Mixer):
     def forward(self, x, batch, cache: CacheView):
         T, g = batch.num_tokens, cache.group
         D2 = 2 * self.dim
+        heads = 2 * self.heads if self.mfma else self.heads       # on the matrix cores a map is a head
+        q_size = heads * D2
         self.qkv.forward(x, self.qkv_buf, T, scratch=True)
         # biases, and the keys and values into their pages: no norm, no rotation
-        ops.qkv_post(self.qkv_buf, T, heads=self.heads, kv_heads=self.kv_heads, head_dim=D2, q_off=0, k_off=self.q_size,
-                     v_off=self.q_size + self.k_size, positions=batch.positions, page_size=self.page_size, q_gain=None,
+        ops.qkv_post(self.qkv_buf, T, heads=heads, kv_heads=self.kv_heads, head_dim=D2, q_off=0, k_off=q_size,
+                     v_off=q_size + self.k_size, positions=batch.positions, page_size=self.page_size, q_gain=None,
                      k_gain=None, eps=0.0, gain_offset=0.0, cos_sin=None, rotary_dim=0, rope_style=0, k_cache=cache.k,
                      v_cache=cache.v, slot_mapping=batch.slot_mapping[g] if cache.owner else None, token_runs=False,
                      v_dim=self.vdim, bias=self.bias_vec)
+        if self.mfma:
+            ops.attn_flash_ext(self.qkv_buf, self.pair_buf, cache.k, cache.v, batch.block_table[g], batch.cu_seqlens,
+                               batch.seq_lens, batch.num_reqs, batch.max_q_len, scale=self.scale, window=self.window or 0,
+                               heads=heads, kv_heads=self.kv_heads, head_dim=D2, page_size=self.page_size, keep_first=0,
+                               sinks=None, slope_exp=0.0, out_scale=1.0)
+            ops.diff_combine(self.pair_buf, self.attn_buf, T, heads=self.heads, v_dim=self.vdim, lam=self.lam,
+                             eps=self.norm_eps, post=1.0 - self.diff)
+            return self.o.forward(self.attn_buf, self.out_buf, T, scratch=True)
         ops.attn_paged_diff(self.qkv_buf, self.attn_buf, cache.k, cache.v, batch.block_table[g], batch.cu_seqlens,
                             batch.seq_lens, batch.num_reqs, T, scale=self.scale, window=self.window or 0,
                             heads=self.heads, kv_heads=self.kv_heads, head_dim=self.dim, v_dim=self.vdim,

@@ -426,8 +426,10 @@ def test_which_kernels_serve_which_model(models):
         mixers = [b.mixer for b in r.model.blocks]
         lefts = [m for mx in mixers if hasattr(mx, "members") for _, m, _, _ in mx.members if hasattr(m, "mfma_ext")]
         latents = [m for m in mixers if hasattr(m, "attn_ws") and hasattr(m, "rank")]
-        assert lefts and latents
+        maps = [m for m in mixers if hasattr(m, "lam")]
+        assert lefts and latents and maps
         assert all(m.mfma_ext == mfma for m in lefts) and all(bool(m.attn_ws.mfma) == mfma for m in latents)
+        assert all(m.mfma == mfma for m in maps)       # (V2: values that are not twice a map's keys wide)
 
 
 def test_layers_that_share_weights_have_caches_of_their_own(models):
