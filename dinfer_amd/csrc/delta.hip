@@ -398,7 +398,8 @@ template <class S>
 __global__ void __launch_bounds__(WAVES * 64) channel_delta_prep_kernel(
     const S* __restrict__ proj, int64_t ld, int64_t r_off, int64_t k_off, int64_t v_off, int64_t a_off, int64_t l_off,
     const float* __restrict__ a_bias, const float* __restrict__ w2, const float* __restrict__ w0, int low,
-    float* __restrict__ work, int64_t ldw, int H, int D, float eps, float rate) {
+    float* __restrict__ work, int64_t ldw, int H, int D, float eps, float rate, const float* __restrict__ z_in,
+    int64_t ld_z) {
   __shared__ float th[WAVES][MAX_LOW];
   const int t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -407,9 +408,11 @@ __global__ void __launch_bounds__(WAVES * 64) channel_delta_prep_kernel(
   const S* row = proj + (int64_t)t * ld;
   float* out = work + (int64_t)t * ldw;
   const int HD = H * D;
-  for (int l = lane; l < low; l += 64) th[wave][l] = tanhf(to_f32(row[l_off + l]));
-  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-  __builtin_amdgcn_wave_barrier();
+  if (!z_in) {
+    for (int l = lane; l < low; l += 64) th[wave][l] = tanhf(to_f32(row[l_off + l]));
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
   constexpr int PER = MAX_HEAD / 64;
   float kk[PER];
   float ss = 0.f;
@@ -430,8 +433,12 @@ __global__ void __launch_bounds__(WAVES * 64) channel_delta_prep_kernel(
       const float u = kk[e] * inv;
       const float a = sigmoid_f(to_f32(row[a_off + c]) + a_bias[c]);
       float z = w0[c];
-      const float* w2r = w2 + (int64_t)c * low;
-      for (int l = 0; l < low; ++l) z = __builtin_fmaf(w2r[l], th[wave][l], z);
+      if (z_in) {   // the product with W2 was a matrix product of its own (steps of many rows)
+        z += z_in[(int64_t)t * ld_z + c];
+      } else {
+        const float* w2r = w2 + (int64_t)c * low;
+        for (int l = 0; l < low; ++l) z = __builtin_fmaf(w2r[l], th[wave][l], z);
+      }
       const float w = expf(-rate * sigmoid_f(z));
       const float au = a * u;
       out[c] = r * w;
@@ -636,18 +643,21 @@ extern "C" int dinfer_delta_out(int dtype, const float* o, int64_t ld_o, const v
 
 // The rule with a decay and a removal rate a key channel (see above). proj [T, ld]: r, k, v (H D each) at their columns,
 // the H D removal logits at a_off, the `low` entries of the decay's inner projection at l_off. a_bias, w0 [H D] float,
-// w2 [H D, low] float. work [T, ldw] float, ldw >= 6 H D + 2 H.
+// w2 [H D, low] float. work [T, ldw] float, ldw >= 6 H D + 2 H. z (may be null) [T, ld_z] float: W2 tanh(.) as a
+// matrix product of the caller's made it; then the kernel only adds w0.
 extern "C" int dinfer_channel_delta_prep(int dtype, const void* proj, int64_t ld, int64_t r_off, int64_t k_off,
                                          int64_t v_off, int64_t a_off, int64_t l_off, const float* a_bias,
                                          const float* w2, const float* w0, int low, float* work, int64_t ldw,
-                                         int64_t tokens, int H, int D, float eps, float rate, hipStream_t stream) {
+                                         int64_t tokens, int H, int D, float eps, float rate, const float* z,
+                                         int64_t ld_z, hipStream_t stream) {
   if (tokens <= 0) return OK;
   if (H <= 0 || D <= 0 || low <= 0 || tokens > 0x7fffffff || ldw < 6LL * H * D + 2 * H) return ERR_BAD_SHAPE;
   if (D > MAX_HEAD || low > MAX_LOW) return ERR_UNSUPPORTED;
   const dim3 grid((unsigned)tokens, (unsigned)((H + WAVES - 1) / WAVES));
   DINFER_DISPATCH_DTYPE(dtype, {
     channel_delta_prep_kernel<S><<<grid, WAVES * 64, 0, stream>>>((const S*)proj, ld, r_off, k_off, v_off, a_off, l_off,
-                                                                  a_bias, w2, w0, low, work, ldw, H, D, eps, rate);
+                                                                  a_bias, w2, w0, low, work, ldw, H, D, eps, rate, z,
+                                                                  ld_z);
   });
   return launch_status();
 }

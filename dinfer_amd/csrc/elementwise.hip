@@ -124,8 +124,9 @@ __global__ void __launch_bounds__(256) embedding_to_kernel(const int32_t* __rest
 }
 
 // Activations of one argument: 0 silu, 1 the square of relu, 2 gelu in its tanh form, 3 gelu with the error function,
-// 4 the logistic function.
+// 4 the logistic function, 5 the hyperbolic tangent.
 __device__ __forceinline__ float act1(float z, int act) {
+  if (act == 5) return tanhf(z);
   if (act == 0) return z / (1.f + expf(-z));
   if (act == 1) { const float r = fmaxf(z, 0.f); return r * r; }
   if (act == 3) return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
@@ -157,6 +158,23 @@ __global__ void __launch_bounds__(256) gated_any_kernel(const S* __restrict__ in
   const int64_t t = blockIdx.y;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < inter; i += (int64_t)gridDim.x * blockDim.x)
     out[t * inter + i] = from_f32<S>(act1(to_f32(in[t * ld_in + i]), act) * to_f32(in[t * ld_in + inter + i]));
+}
+
+// The same, 8 bf16 per thread and iteration; needs inter % 8 == 0 and 16-byte aligned rows.
+__global__ void __launch_bounds__(256) gated_any_bf16x8_kernel(const bf16* __restrict__ in, bf16* __restrict__ out,
+                                                               int64_t inter, int64_t ld_in, int act) {
+  const int64_t t = blockIdx.y;
+  const bf16x8* g = (const bf16x8*)(in + t * ld_in);
+  const bf16x8* u = (const bf16x8*)(in + t * ld_in + inter);
+  bf16x8* o = (bf16x8*)(out + t * inter);
+  const int64_t n8 = inter / 8;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += (int64_t)gridDim.x * blockDim.x) {
+    const bf16x8 gv = g[i], uv = u[i];
+    bf16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = (bf16)(act1((float)gv[j], act) * (float)uv[j]);
+    o[i] = r;
+  }
 }
 
 // Token shift: out[t] = x[t] + (before - x[t]) * mix, `before` the row of the token before in its request: the row
@@ -215,6 +233,11 @@ extern "C" int dinfer_gated_act(int dtype, int act, const void* in, void* out, i
     for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
       const int64_t nt = tokens - t0 < 65535 ? tokens - t0 : 65535;
       const dim3 grid(blocks_for(inter, 256, 64), (unsigned)nt);
+      if (dtype == DT_BF16 && inter % 8 == 0 && ld_in % 8 == 0 && ((uintptr_t)in % 16 == 0) && ((uintptr_t)out % 16 == 0)) {
+        gated_any_bf16x8_kernel<<<dim3(blocks_for(inter / 8, 256, 64), (unsigned)nt), 256, 0, stream>>>(
+            (const bf16*)in + t0 * ld_in, (bf16*)out + t0 * inter, inter, ld_in, act);
+        continue;
+      }
       DINFER_DISPATCH_DTYPE(dtype, {
         gated_any_kernel<S><<<grid, 256, 0, stream>>>((const S*)in + t0 * ld_in, (S*)out + t0 * inter, inter, ld_in, act);
       });
@@ -314,7 +337,7 @@ extern "C" int dinfer_gate(int dtype, int act, void* x, int64_t ld_x, const void
 extern "C" int dinfer_act(int dtype, int act, const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t tokens,
                           int64_t n, hipStream_t stream) {
   if (tokens <= 0 || n <= 0) return OK;
-  if (act < 0 || act > 4) return ERR_UNSUPPORTED;
+  if (act < 0 || act > 5) return ERR_UNSUPPORTED;
   if (ld_in < n || ld_out < n) return ERR_BAD_SHAPE;
   for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
     const int64_t nt = tokens - t0 < 65535 ? tokens - t0 : 65535;
@@ -325,6 +348,52 @@ extern "C" int dinfer_act(int dtype, int act, const void* in, int64_t ld_in, voi
   }
   return launch_status();
 }
+
+namespace {
+// The same with 8 bf16 a thread (16-byte loads and stores): width % 8 == 0, rows and state 16-byte aligned. A thread
+// keeps its 8 channels' shares and walks the workgroup's rows; grid.z cuts the width where a workgroup does not span it.
+__global__ void __launch_bounds__(256) token_shift_bf16x8_kernel(const bf16* __restrict__ x, int64_t ld_x,
+                                                                 bf16* __restrict__ out, int64_t ld_out,
+                                                                 bf16* __restrict__ state, const float* __restrict__ mix,
+                                                                 const int32_t* __restrict__ cu,
+                                                                 const int32_t* __restrict__ seq_lens,
+                                                                 const int32_t* __restrict__ slots, int64_t width) {
+  const int b = blockIdx.y;
+  const int t0 = cu[b], n = cu[b + 1] - t0;
+  const int r0 = blockIdx.x * SHIFT_TOK;
+  const int64_t i = ((int64_t)blockIdx.z * blockDim.x + threadIdx.x) * 8;
+  if (r0 >= n || i >= width) return;
+  const bool starts = seq_lens[b] - n <= 0;
+  const int r1 = r0 + SHIFT_TOK < n ? r0 + SHIFT_TOK : n;
+  bf16* kept = state + (int64_t)slots[b] * width + i;
+  const f32x4 m0 = *(const f32x4*)(mix + i), m1 = *(const f32x4*)(mix + i + 4);
+  float m[8] = {m0[0], m0[1], m0[2], m0[3], m1[0], m1[1], m1[2], m1[3]};
+  bf16x8 before;
+  if (r0 > 0) before = *(const bf16x8*)(x + (int64_t)(t0 + r0 - 1) * ld_x + i);
+  else if (starts) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) before[j] = (bf16)0.f;
+  } else before = *(const bf16x8*)kept;
+  // all rows' loads first: they do not depend on each other
+  bf16x8 rows[SHIFT_TOK];
+#pragma unroll
+  for (int r = 0; r < SHIFT_TOK; ++r)
+    if (r0 + r < r1) rows[r] = *(const bf16x8*)(x + (int64_t)(t0 + r0 + r) * ld_x + i);
+#pragma unroll
+  for (int r = 0; r < SHIFT_TOK; ++r) {
+    if (r0 + r >= r1) break;
+    bf16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float v = (float)rows[r][j];
+      o[j] = (bf16)(v + ((float)before[j] - v) * m[j]);
+    }
+    *(bf16x8*)(out + (int64_t)(t0 + r0 + r) * ld_out + i) = o;
+    before = rows[r];
+  }
+  if (r0 == 0) *(bf16x8*)kept = *(const bf16x8*)(x + (int64_t)(t0 + n - 1) * ld_x + i);
+}
+}  // namespace
 
 // out[t] = x[t] + (row before - x[t]) * mix for the rows of num_reqs requests (cu_seqlens), the row before a
 // portion's first row taken from state[slots[b]] (zeros for a request that starts), which then takes the portion's
@@ -337,6 +406,14 @@ extern "C" int dinfer_token_shift(int dtype, const void* x, int64_t ld_x, void* 
   if (num_reqs <= 0 || max_rows <= 0) return OK;
   if (width <= 0 || ld_x < width || ld_out < width || num_reqs > 65535 || x == out) return ERR_BAD_SHAPE;
   const dim3 grid((unsigned)((max_rows + SHIFT_TOK - 1) / SHIFT_TOK), (unsigned)num_reqs);
+  if (dtype == DT_BF16 && width % 8 == 0 && ld_x % 8 == 0 && ld_out % 8 == 0 && ((uintptr_t)x % 16 == 0) &&
+      ((uintptr_t)out % 16 == 0) && ((uintptr_t)state % 16 == 0) && ((uintptr_t)mix % 16 == 0)) {
+    const int threads = width >= 2048 ? 256 : width >= 512 ? 64 * (int)((width / 8 + 63) / 64) : 64;
+    const dim3 vgrid(grid.x, grid.y, (unsigned)((width / 8 + threads - 1) / threads));
+    token_shift_bf16x8_kernel<<<vgrid, threads, 0, stream>>>((const bf16*)x, ld_x, (bf16*)out, ld_out, (bf16*)state, mix,
+                                                             cu_seqlens, seq_lens, slots, width);
+    return launch_status();
+  }
   DINFER_DISPATCH_DTYPE(dtype, {
     token_shift_kernel<S><<<grid, width >= 256 ? 256 : 64, 0, stream>>>((const S*)x, ld_x, (S*)out, ld_out, (S*)state, mix,
                                                                         cu_seqlens, seq_lens, slots, width);

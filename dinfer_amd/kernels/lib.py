@@ -65,7 +65,8 @@ SIGNATURES = {
     "dinfer_delta_conv_update": ("delta", [_I, _P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _P]),
     "dinfer_delta_recurrence": ("delta", [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P]),
     "dinfer_delta_out": ("delta", [_I, _P, _L, _P, _L, _L, _P, _P, _L, _L, _L, _I, _I, _F, _F, _I, _I, _P]),
-    "dinfer_channel_delta_prep": ("delta", [_I, _P, _L, _L, _L, _L, _L, _L, _P, _P, _P, _I, _P, _L, _L, _I, _I, _F, _F, _P]),
+    "dinfer_channel_delta_prep": ("delta", [_I, _P, _L, _L, _L, _L, _L, _L, _P, _P, _P, _I, _P, _L, _L, _I, _I, _F, _F, _P, _L,
+                                            _P]),
     "dinfer_channel_delta_recurrence": ("delta", [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P]),
     "dinfer_gate": ("elementwise", [_I, _I, _P, _L, _P, _L, _L, _L, _L, _P]),
     "dinfer_token_shift": ("elementwise", [_I, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _L, _L, _P]),

@@ -155,7 +155,7 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float
 
 
 # activations of one argument -> their code in the C interface ("gelu": with the error function)
-ACTS = {"silu": 0, "relu2": 1, "gelu_tanh": 2, "gelu": 3, "sigmoid": 4}
+ACTS = {"silu": 0, "relu2": 1, "gelu_tanh": 2, "gelu": 3, "sigmoid": 4, "tanh": 5}
 
 
 def act(x: torch.Tensor, out: torch.Tensor, tokens: int, kind: str) -> torch.Tensor:
@@ -372,10 +372,13 @@ def channel_delta_work_columns(heads: int, dim: int) -> int:
 
 def channel_delta_prep(proj: torch.Tensor, tokens: int, *, r_off: int, k_off: int, v_off: int, a_off: int, low_off: int,
                        a_bias: torch.Tensor, w2: torch.Tensor, w0: torch.Tensor, work: torch.Tensor, heads: int, dim: int,
-                       eps: float, rate: float) -> None:
+                       eps: float, rate: float, z: torch.Tensor | None = None) -> None:
     """From the step's projections: the unit key u = k / sqrt(sum k^2 + eps), the removal rate a = sigmoid(. + a_bias),
-    the decay w = exp(-rate * sigmoid(w2 tanh(low) + w0)), and what the recurrence reads of them, in float32."""
-    _need_gpu(proj, a_bias, w2, w0, work)
+    the decay w = exp(-rate * sigmoid(w2 tanh(low) + w0)), and what the recurrence reads of them, in float32.
+    z: float32 [T, heads * dim], w2 tanh(low) where the caller has made it by a matrix product of its own."""
+    _need_gpu(proj, a_bias, w2, w0, work, z)
+    if z is not None:
+        assert z.dtype == torch.float32 and z.shape[0] >= tokens and z.shape[1] >= heads * dim
     hd = heads * dim
     low = w2.shape[1]
     assert a_bias.dtype == w2.dtype == w0.dtype == torch.float32 and w2.is_contiguous()
@@ -384,7 +387,7 @@ def channel_delta_prep(proj: torch.Tensor, tokens: int, *, r_off: int, k_off: in
     assert proj.shape[0] >= tokens and max(r_off, k_off, v_off, a_off) + hd <= proj.shape[1] and low_off + low <= proj.shape[1]
     lib.call("dinfer_channel_delta_prep", dtype_code(proj.dtype), proj.data_ptr(), _rows(proj), r_off, k_off, v_off, a_off,
              low_off, a_bias.data_ptr(), w2.data_ptr(), w0.data_ptr(), low, work.data_ptr(), _rows(work), tokens, heads,
-             dim, float(eps), float(rate), _stream())
+             dim, float(eps), float(rate), _ptr(z), _rows(z) if z is not None else 0, _stream())
 
 
 def channel_delta_recurrence(work: torch.Tensor, state: torch.Tensor, out: torch.Tensor, *, state_slots: torch.Tensor,

@@ -11,9 +11,11 @@ With h the mixer's input, H heads of `dim` entries:
     y = Wo ( concat_h( o_h / rms(o_h) ) * g * sigmoid(Wg h) )                          (g: a gain of H dim entries)
 
 One product makes r | k | v | gate | removal logits | Ww1 h; what follows up to the operand of Wo is float
-(csrc/delta.hip). The state lives in the request's state slot (DeltaStateSpec without a convolution); a request's
-first step (position 0) starts from zeros. Prompt portions of any size and single rows run the same kernels and leave
-the same bits.
+(csrc/delta.hip). The small product with Ww2 rides in the kernel that prepares the recurrence in steps of few rows;
+in steps of many it is a matrix product of its own (tanh in the engine's dtype, the result float32). The state lives in the request's state slot (DeltaStateSpec without a convolution); a request's
+first step (position 0) starts from zeros. Prompt portions of any size and single rows run the same recurrence, every
+token the same arithmetic in the same order; only the decay's inner product is summed in another order in steps of
+many rows.
 """
 from __future__ import annotations
 
@@ -21,13 +23,17 @@ import math
 
 import torch
 
-from ..kernels import ops
+from ..kernels import gemm, ops
 from .base import CacheView, Mixer
 from .linear import Linear
 from .registry import MIXERS
 from .spec import DeltaStateSpec, TensorSpec
 
 DEFAULT_RATE = math.exp(-0.5)
+# Up to this many rows the product with Ww2 rides in the preparing kernel (a wave a (token, head) reads the head's rows
+# of Ww2: two launches fewer); beyond, every wave reading them again costs more than a matrix product (2,048 rows of 32
+# heads of 64 with 64 inside: 147 us against 20 for the act and the product)
+LOW_IN_KERNEL_ROWS = 64
 
 
 @MIXERS.register("channel_delta_rule")
@@ -88,6 +94,7 @@ class ChannelDeltaRule(Mixer):
         # small parameters in 32 bits (exact for a bfloat16 file): they enter the recurrence
         self.a_bias = get(n["a_bias"]).float().contiguous()
         self.w2 = get(n["w2"]).float().contiguous()
+        self.w2_operand = get(n["w2"], compute=True).contiguous()
         self.w0 = get(n["w0"]).float().contiguous()
         self.norm_weight = get(n["norm"]).float().contiguous()
 
@@ -107,6 +114,8 @@ class ChannelDeltaRule(Mixer):
         ws = ctx.workspace
         self.work = ws.buffer("channel_delta_work", ops.channel_delta_work_columns(self.heads, self.dim), dtype=torch.float32)
         self.o_buf = ws.buffer("channel_delta_o", self.size, dtype=torch.float32)
+        self.tanh_buf = ws.buffer("channel_delta_tanh", self.low)
+        self.z_buf = ws.buffer("channel_delta_z", self.size, dtype=torch.float32)
 
     def forward(self, x, batch, cache: CacheView):
         T = batch.num_tokens
@@ -120,10 +129,15 @@ class ChannelDeltaRule(Mixer):
         T = batch.num_tokens
         if not cache.owner:
             raise NotImplementedError("a recurrent mixer keeps a state a request: an entry that borrows a cache has none")
+        z = None
+        if T > LOW_IN_KERNEL_ROWS:
+            lo = col + self.l_off
+            ops.act(proj_buf[:, lo:lo + self.low], self.tanh_buf, T, "tanh")
+            z = gemm.matmul_nt(self.tanh_buf, self.w2_operand, self.z_buf, T, may_pad=True)
         ops.channel_delta_prep(proj_buf, T, r_off=col, k_off=col + self.k_off, v_off=col + self.v_off,
                                a_off=col + self.a_off, low_off=col + self.l_off, a_bias=self.a_bias, w2=self.w2,
                                w0=self.w0, work=self.work, heads=self.heads, dim=self.dim, eps=self.unit_eps,
-                               rate=self.rate)
+                               rate=self.rate, z=z)
         ops.channel_delta_recurrence(self.work, cache.state, self.o_buf, state_slots=batch.state_slots,
                                      cu_seqlens=batch.cu_seqlens, seq_lens=batch.seq_lens, num_reqs=batch.num_reqs,
                                      heads=self.heads, dim=self.dim)
