@@ -76,6 +76,8 @@ ONE = {
     "latent": (model(64, 32, [dense(L1, None)]), 4, 21),
     "differential": (model(64, 32, [dense(D1, None)]), 4, 22),
     "left": (model(64, 32, [dense(parallel(4, 2, 16, 8, 6, 8, 2, 8, 1.0, 0.0), None)]), 4, 23),
+    # bfloat16: heads of 64 rotated whole, which the 16-byte kernel before the cache takes (with the temperature)
+    "left_whole": (model(64, 48, [dense(parallel(4, 2, 64, 64, 6, 64, 1, 8, 1.0, 0.0), None)]), 8, 27),
     "right": (model(64, 32, [dense(parallel(2, 1, 8, 8, 6, 4, 4, 24, 0.0, 1.0), None)]), 4, 24),
     "dense": (model(64, 32, [dense(parallel(2, 1, 8, 8, 6, 4, 2, 8, 0.0, 0.0), 72)]), 4, 25),
     "routed": (model(64, 32, [routed(parallel(2, 1, 8, 8, 6, 4, 2, 8, 0.0, 0.0), 7, 2, 3, 24)]), 4, 26),
