@@ -719,3 +719,39 @@ def test_trace_replay_program(models, tmp_path, dtype):
     for step, wanted in ((0, [("a", 3), ("a", 24)]), (1, [("a", 25), ("b", 8)]), (2, [("a", 39)])):
         got = torch.from_numpy(np.fromfile(tmp_path / f"{step}.f32", dtype="<f4").reshape(len(wanted), cfg["vocab"]))
         check_logits(got, torch.stack([full[k][p] for k, p in wanted]), dtype, f"trace step {step}")
+
+
+def test_command_line_writes_random_weights_and_generates(models, tmp_path):
+    """bin/dinfer random-weights from a configuration that names the decay projection's inner size, then bin/dinfer
+    generate on that folder and on a folder of the plain model's weights, where the greedy tokens are the plain
+    model's wherever its choice is clear."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    d, cfg, w, page = models["V1"]
+    root = Path(__file__).resolve().parent.parent
+    exe = [sys.executable, str(root / "bin" / "dinfer")]
+    named = copy.deepcopy(cfg)
+    for l in named["layers"]:
+        if l["type"] == "parallel":
+            l["mixer"]["right"]["decay_rank"] = 9
+    (tmp_path / "config.json").write_text(json.dumps(named))
+    p = subprocess.run(exe + ["random-weights", "--config", str(tmp_path / "config.json"), "--out", str(tmp_path / "m"), "--seed", "3"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    common = ["--dtype", "float32", "--max-model-len", "128", "--max-num-seqs", "2", "--num-blocks", "64", "--block-size", str(page),
+              "--max-num-batched-tokens", "64", "--max-tokens", "8", "--temperature", "0", "--prompt-ids", "5,9,2", "--prompt-ids", "7"]
+    p = subprocess.run(exe + ["generate", "--model", str(tmp_path / "m")] + common, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    recs = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
+    assert [r["prompt_ids"] for r in recs] == [[5, 9, 2], [7]] and all(len(r["output_ids"]) == 8 for r in recs)
+    p = subprocess.run(exe + ["generate", "--model", str(d)] + common, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    for r in (json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")):
+        ids = list(r["prompt_ids"])
+        for tok in r["output_ids"]:
+            logits = plain.forward(ids, w, cfg)[-1]
+            top2 = logits.topk(2).values
+            if (top2[0] - top2[1]).item() > 1e-3 * logits.std().item():
+                assert tok == int(logits.argmax())
+            ids.append(tok)
