@@ -14,7 +14,9 @@ config.json is nested; every size and every constant that may differ between mod
                     parallel:         left{heads, kv_heads, dim, vdim, scale, mask{size}, rot{base, dims}},
                                       right{heads, dim}, left_scale, right_scale
     layers[i].mlp   null | {kind: "dense", ff} | {kind: "moe", expert{ff}, router{experts, identity, top}}
-    layers[i].weights_of   (optional) j: the layer has no tensors and runs on layer j's, with a cache of its own
+    layers[i].weights_of   (optional) j: the layer has no tensors and runs on layer j's, with a cache of its own (its entry
+                    is expected to equal layer j's; where a constant differs, a window say, the entry's own counts, and
+                    a size that does not fit layer j's tensors is refused when the weights are checked)
 
 One size is in no key: the inner size of the decay projection of a parallel layer's right half is the row count of the
 tensor l<i>.mix.right.w1. `sizes_from_tensors` puts it into the parsed file as right.decay_rank before the
@@ -211,8 +213,9 @@ class VeroraxConfig(ModelConfig):
             out.append(VeroraxLayer(typ, _mixer(typ, _section(l, "mixer", where), where + "mixer."),
                                     _feed_forward(l.get("mlp"), where), src))
         for i, l in enumerate(out):
-            if l.weights_of is not None and (l.mixer, l.mlp) != (out[l.weights_of].mixer, out[l.weights_of].mlp):
-                raise ConfigError(f"config key layers[{i}]: a layer with 'weights_of' has the sizes of the layer it names")
+            if l.weights_of is not None and (l.mlp is None) != (out[l.weights_of].mlp is None):
+                raise ConfigError(f"config key layers[{i}]: a layer with 'weights_of' has a feed-forward if and only if the "
+                                  "layer it names has one")
         return {"norm_eps": _num(_section(d, "norm", ""), "eps", float, "norm."), "layers": tuple(out)}
 
     def check(self) -> None:

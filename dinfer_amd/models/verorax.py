@@ -9,7 +9,8 @@ per-head q/k norm, a rotation of part of each head, a temperature a head and one
 rule with a decay and a removal rate a key channel; the two scaled and summed). Rotations pair entry i with
 i + dims/2. Feed-forwards: gated with the tanh form of gelu, or routed experts (silu) chosen by softmax score plus a
 correction, weighted by the scores as they are, the last router outputs standing for experts that hand their input
-on. A layer with `weights_of` is a second run entry of the layer it names, with a cache of its own.
+on. A layer with `weights_of` is a second run entry of the layer it names, with a cache of its own (where its entry
+differs from that layer's in a constant, it is a layer of its own that reads the same tensors).
 Tensor names: embed, l<i>.norm{1,1b,2,2b}, l<i>.shift, l<i>.mix.{dq, dq.norm, uq, dkv, dkv.norm, uk, uv, o} or
 l<i>.mix.{q, k, v}(.b), l<i>.mix.{lq1, lk1, lq2, lk2, o} or l<i>.mix.left.{q, k, v, q.norm, k.norm, temp, g, o} and
 l<i>.mix.right.{r, k, v, g, a, a.b, w1, w2, w0, norm, o}; l<i>.mlp.{gate, up, down} or
@@ -68,7 +69,14 @@ def build_spec(cfg: VeroraxConfig) -> ModelSpec:
             layers.append(LayerSpec(block=part("sandwich", shift="shift"), mixer=_mixer(cfg, l),
                                     feed_forward=_feed_forward(l.mlp), norm=norm, prefix=f"l{i}."))
     for i, l in enumerate(cfg.layers):
-        run.append(RunEntry(place[i if l.weights_of is None else l.weights_of]))
+        src = i if l.weights_of is None else l.weights_of
+        if src != i and (l.mixer, l.mlp) != (cfg.layers[src].mixer, cfg.layers[src].mlp):
+            # the same tensors under constants of its own (a window, a scale): a layer of its own that reads them again
+            place[i] = len(layers)
+            layers.append(LayerSpec(block=part("sandwich", shift="shift"), mixer=_mixer(cfg, l),
+                                    feed_forward=_feed_forward(l.mlp), norm=norm, prefix=f"l{src}."))
+            src = i
+        run.append(RunEntry(place[src]))
     return ModelSpec(
         architecture=cfg.ARCHITECTURE, vocab_size=cfg.vocab, hidden_size=cfg.width, max_positions=cfg.MAX_POSITIONS,
         layers=layers, run=run, final_norm=norm, final_norm_name="final.norm", embed_name="embed", head_name="head",

@@ -69,7 +69,10 @@ CONFIGS = {
     # the model starts with layers that share weights; sizes the matrix-core kernels take; pages of 16
     "V3": (model(120, 128, [dense(P3, 96), shared(dense(P3, 96), 0), routed(L3, 8, 2, 2, 64), dense(D3, 64),
                             shared(dense(D3, 64), 3)]), 16, 13),
-    "V4": (model(77, 40, [dense(P4, 56), dense(D1, 24)]), 4, 14),
+    # the second layer runs on the first's weights with another window and another diff, the fourth on the third's
+    # with another scale and other shares of its halves
+    "V4": (model(77, 40, [dense(D1, 24), dict(shared(dense(differential(4, 2, 8, 16, size=3, diff=0.5), 24), 0)),
+                          dense(P4, 56), shared(dense(parallel(6, 3, 8, 4, 9, 2, 1, 64, 0.3, 1.1, scale=0.5), 56), 2)]), 4, 14),
 }
 # one mechanism a model (a parallel layer's other half scaled by zero)
 ONE = {
@@ -624,12 +627,12 @@ def test_a_key_far_back_among_hundreds(models, dtype):
 
 
 def test_pages_behind_the_window_are_given_back(models):
-    _, cfg, w, page = models["V4"]      # windows 3 and 10, pages of 4: every layer's pages are given back
+    _, cfg, w, page = models["V4"]      # windows 10, 3, 3 and 9, pages of 4: every layer's pages are given back
     r = make_runner(models, "V4", "float32", num_blocks=110, max_len=400)
     ids = tokens_for(cfg, 300, 4)
     rows = replay(r, [([("x", p, [len(p) - 1])], []) for p in cut(ids, [9, 1, 1, 30, 2])])
     compare_rows(rows, cfg, w, {"x": ids}, "float32", "V4 long request")
-    assert len(r.group_specs) == 2
+    assert len(r.group_specs) == 4
     for g, spec in enumerate(r.group_specs):
         held = [i for i, pg in enumerate(r.cache.block_table("x", g)) if pg >= 0]
         assert held == list(range((len(ids) - spec.window + 1) // page, (len(ids) - 1) // page + 1))

@@ -65,10 +65,8 @@ def test_config_round_trip_and_refusals():
     for change in bad:
         with pytest.raises(ConfigError):
             parsed(config(**change))
-    other = copy.deepcopy(latent())
-    other["mixer"]["heads"] = 2
-    with pytest.raises(ConfigError):                    # a layer on another's weights has that layer's sizes
-        parsed(config(layers=[latent(), dict(other, weights_of=0)]))
+    with pytest.raises(ConfigError):                    # a layer on another's weights has a feed-forward if that one has
+        parsed(config(layers=[latent(), dict(latent(), mlp=None, weights_of=0)]))
     with pytest.raises(ConfigError):                    # the decay projection's inner size is in no key and no tensor
         parsed(config(rank=None))
 
@@ -99,6 +97,22 @@ def test_run_order_tensor_names_and_caches():
     shapes = plain.tensor_shapes(config(rank=6))
     assert {n: tuple(s.shape) for n, s in exp.items()} == {n: tuple(s) for n, s in shapes.items()}
     assert not any(n.startswith("l3.") for n in exp)
+
+
+def test_a_layer_on_anothers_weights_with_constants_of_its_own():
+    """Equal entries share one layer of the description; an entry that differs in a constant becomes a layer of its own
+    under the same tensor names, and a size that does not fit those tensors is left to the check of the weights."""
+    from dinfer_amd.parts import DecoderModel
+    other = differential()
+    other["mixer"]["mask"]["size"] = 4
+    other["mixer"]["diff"] = 0.5
+    cfg = config(layers=[differential(), dict(differential(), weights_of=0), dict(other, weights_of=0)])
+    arch, c = parsed(cfg)
+    spec = arch.build_spec(c)
+    assert [e.layer for e in spec.run] == [0, 0, 1] and [l.prefix for l in spec.layers] == ["l0.", "l0."]
+    assert spec.layers[1].mixer.params["window"] == 4 and spec.layers[0].mixer.params["window"] == 9
+    exp, _ = DecoderModel(spec).expected_tensors()
+    assert set(exp) == set(plain.tensor_shapes(cfg))
 
 
 def test_token_shift_by_hand():
